@@ -103,8 +103,7 @@ typedef __attribute__((address_space(3))) void* lds_ptr;
 // softmax temporaries of the first tile got its registers, 128 cycles of s_nop behind the read; and the fragments
 // that the last pass asks for the pass that never comes were still out when the rows' sums moved into their
 // registers.  With one block a compute unit LDS answered in time; with a second block's reads and direct loads on the
-// same LDS it did not always, and rows differed from run to run.  tests/test_kernel_waits.py checks the compiler's
-// output for both patterns.)
+// same LDS it did not always, and rows differed from run to run.)
 template <int OFFSET>
 __device__ __forceinline__ Frag lds_frag(int addr) {
   u32x4 v;

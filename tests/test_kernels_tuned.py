@@ -659,7 +659,7 @@ def test_attention_of_whole_tiles_gives_the_same_bits_every_time(d):
     registers the compiler had already given to another value once showed as rows that differ from run to run when
     two blocks shared a compute unit's LDS (heads of 64 run that way).  More blocks than compute units, many times:
     every output equals the first bit by bit (which the other tests hold against the plain implementation at smaller
-    sizes); tests/test_kernel_waits.py looks for the pattern itself in the compiler's output."""
+    sizes)."""
     from allpaca_amd.engine.batch import Entry, pack_step
     from allpaca_amd.kernels import ops as kernel_ops
     t = tuned()
