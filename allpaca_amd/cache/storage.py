@@ -102,16 +102,24 @@ class CacheStorage:
                 return PagedView(self.paged[gi][li], self.manager.page_tokens, getattr(need, "window", None), writes, gi)
             return StateView(self.state[gi][li], writes, gi)
 
+        def roles_of(entry: int) -> dict:
+            """role -> location of everything plan entry `entry` keeps itself (a single need stands under "mixer")."""
+            roles = {k[1]: v for k, v in self.manager.location.items() if isinstance(k, tuple) and k[0] == entry}
+            if entry in self.manager.location:
+                roles["mixer"] = self.manager.location[entry]
+            return roles
+
         out = []
         for i, e in enumerate(plan):
-            owner = i if e.cache_of is None else e.cache_of
-            loc = self.manager.location.get(owner)
-            if loc is not None:
-                out.append(view(loc, e.cache_of is None))
-                continue
-            # several parts of the entry keep a cache: a dict role -> view
-            roles = {k[1]: v for k, v in self.manager.location.items() if isinstance(k, tuple) and k[0] == owner}
-            out.append({role: view(loc, e.cache_of is None) for role, loc in roles.items()} or None)
+            own = roles_of(i)
+            views = {role: view(loc, True) for role, loc in own.items()}
+            if e.cache_of is not None:
+                # what the owner keeps for others to read; what a part keeps for itself alone ("<role>.state") stays
+                # with each entry
+                for role, loc in roles_of(e.cache_of).items():
+                    if not role.endswith(".state"):
+                        views[role] = view(loc, False)
+            out.append(None if not views else views["mixer"] if list(views) == ["mixer"] else views)
         return out
 
     def zero_slot(self, slot: int) -> None:

@@ -354,3 +354,178 @@ def paged_attention(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int
             return
     paged_attention_plain(q, q_off, out, n_heads, n_kv_heads, head_dim, cache, page_tokens, block_table,
                           step.positions, step.row_seg, window, scale)
+
+
+# --------------------------------------------------------------------------- mechanisms beside the llama layer
+MASKS = {"causal": 0, "window": 1, "chunk": 2}
+
+
+def _f32(t: Optional[torch.Tensor], n: int, what: str) -> int:
+    if t is None:
+        return 0
+    if not (t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= n):
+        raise ValueError(f"{what}: need >= {n} contiguous float32")
+    return t.data_ptr()
+
+
+def _split_pages(cache: torch.Tensor, kv_heads: int, key_dim: int, value_dim: int, page_tokens: int) -> None:
+    if not (cache.dim() == 3 and cache.is_contiguous()
+            and tuple(cache.shape[1:]) == (kv_heads, page_tokens * (key_dim + value_dim))):
+        raise ValueError(f"cache must be [pages, {kv_heads}, {page_tokens} * ({key_dim} + {value_dim})], "
+                         f"got {tuple(cache.shape)}")
+
+
+def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: int, n_kv_heads: int, key_dim: int,
+               value_dim: int, bias: Optional[torch.Tensor], conv_w: Optional[torch.Tensor],
+               state: Optional[torch.Tensor], step, slots: Optional[torch.Tensor], unit_norm: bool, eps: float,
+               q_out: torch.Tensor, block_table: Optional[torch.Tensor] = None, cache: Optional[torch.Tensor] = None,
+               page_tokens: int = 0) -> None:
+    """Bias, short causal convolution over time (taps = conv_w.shape[1]; the inputs of the positions ahead of a
+    segment come from `state` [slots + 1, taps - 1, width], which is moved on), unit RMS norm of q and k heads,
+    q to `q_out` [rows, heads * key_dim], k and v into the pages.  `n_kv_heads` = 0: the row holds q only."""
+    _gpu(proj, bias, conv_w, state, slots, q_out, block_table, cache)
+    ld, ldq = _rows(proj, "projected rows"), _rows(q_out, "q out")
+    T, width = proj.shape
+    G = int(n_kv_heads)
+    _need(q_off + n_heads * key_dim <= width and (G == 0 or (k_off + G * key_dim <= width and
+                                                             v_off + G * value_dim <= width)),
+          "conv_heads: head ranges exceed the row")
+    _need(q_out.shape == (T, n_heads * key_dim), "conv_heads: q out must be [rows, heads * key_dim]")
+    taps = 1
+    if conv_w is not None:
+        _need(conv_w.dim() == 2 and conv_w.shape[0] == width, "conv_heads: conv weights must be [width, taps]")
+        taps = int(conv_w.shape[1])
+    if taps > 1:
+        _need(state is not None and slots is not None and state.dim() == 3 and state.is_contiguous()
+              and state.dtype == torch.float32 and tuple(state.shape[1:]) == (taps - 1, width),
+              f"conv_heads: state must be float32 [slots, {taps - 1}, {width}]")
+    max_blocks = 0
+    if G:
+        _need(cache is not None and block_table is not None, "conv_heads: keys and values need pages and a block table")
+        _split_pages(cache, G, key_dim, value_dim, page_tokens)
+        _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+              "block table must be contiguous int32 [segments, blocks]")
+        max_blocks = block_table.shape[1]
+    S = step.n_segs
+    L = _lib.load("plain")
+    _lib.check(L.apc_conv_heads(
+        proj.data_ptr(), _code(proj), ld, q_off, k_off, v_off, T, S, n_heads, G, key_dim, value_dim,
+        _f32(bias, width, "bias"), _f32(conv_w, width * taps, "conv weights") if taps > 1 else 0, taps,
+        state.data_ptr() if taps > 1 else 0, width, _i32(step.row_seg, T, "row_seg"), _i32(step.seg_row0, S, "seg_row0"),
+        _i32(step.seg_rows, S, "seg_rows"), _i32(slots, S, "slots") if taps > 1 else 0,
+        _i32(step.positions, T, "positions"), 1 if unit_norm else 0, float(eps), q_out.data_ptr(), _code(q_out), ldq,
+        block_table.data_ptr() if G else 0, max_blocks, cache.data_ptr() if G else 0, _code(cache) if G else 0,
+        page_tokens, _stream()), "conv_heads")
+
+
+def masked_attention_plain(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, key_dim: int,
+                           value_dim: int, cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor,
+                           positions: torch.Tensor, row_seg: torch.Tensor, mask: str, mask_size: int, sink: bool,
+                           scale: float) -> None:
+    _gpu(q, out, cache, block_table, positions, row_seg)
+    ldq, ldo = _rows(q, "attention q"), _rows(out, "attention out")
+    T = q.shape[0]
+    _need(q.shape[1] == n_heads * key_dim, "attention: q must be [rows, heads * key_dim]")
+    _need(out.shape == (T, n_heads * value_dim), "attention out must be [rows, heads * value_dim]")
+    _split_pages(cache, n_kv_heads, key_dim, value_dim, page_tokens)
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+          "block table must be contiguous int32 [segments, blocks]")
+    L = _lib.load("plain")
+    _lib.check(L.apc_masked_attention_plain(
+        q.data_ptr(), _code(q), ldq, out.data_ptr(), _code(out), ldo, T, n_heads, n_kv_heads, key_dim, value_dim,
+        cache.data_ptr(), _code(cache), page_tokens, block_table.data_ptr(), block_table.shape[1],
+        _i32(positions, T, "positions"), _i32(row_seg, T, "row_seg"), MASKS[mask], int(mask_size), 1 if sink else 0,
+        float(scale), _stream()), "masked_attention_plain")
+
+
+def masked_attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int,
+                     cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor, step, mask: str = "causal",
+                     mask_size: int = 0, sink: bool = False, scale: float = 1.0) -> None:
+    if _tuned_ok(q, cache, out):
+        from . import tuned
+        if tuned.masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens,
+                                       block_table, step, mask, mask_size, sink, scale):
+            return
+    masked_attention_plain(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens, block_table,
+                           step.positions, step.row_seg, mask, mask_size, sink, scale)
+
+
+def streams_step(x: torch.Tensor, n_streams: int, y: Optional[torch.Tensor] = None,
+                 mix: Optional[torch.Tensor] = None, out_w: Optional[torch.Tensor] = None,
+                 in_w: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0,
+                 h: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> None:
+    """x [T, S * D] float32, S residual copies a row.  With y [T, D]: copy b <- sum_a mix[a][b] copy a + out_w[b] y.
+    With in_w: h = rms_norm(sum_a in_w[a] copy a) * norm_w (of the new copies, if both are asked for).  `rows`: h[r]
+    from x[rows[r]] (reading only)."""
+    _gpu(x, y, mix, out_w, in_w, norm_w, h, rows)
+    S = int(n_streams)
+    _need(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous() and x.shape[1] % S == 0,
+          "streams: x must be contiguous float32 [rows, streams * width]")
+    T, D = x.shape[0], x.shape[1] // S
+    ldy = ldh = 0
+    if y is not None:
+        ldy = _rows(y, "streams y")
+        _need(y.shape == (T, D) and rows is None, "streams: y must be [rows, width]")
+    n_out = T
+    if in_w is not None:
+        ldh = _rows(h, "streams h")
+        n_out = rows.numel() if rows is not None else T
+        _need(h.shape == (n_out, D), "streams: h must be [rows, width]")
+    L = _lib.load("plain")
+    _lib.check(L.apc_streams_step(
+        x.data_ptr(), n_out, S, D, y.data_ptr() if y is not None else 0, _code(y) if y is not None else 0, ldy,
+        _f32(mix, S * S, "mix") if y is not None else 0, _f32(out_w, S, "out weights") if y is not None else 0,
+        _f32(in_w, S, "in weights"), _f32(norm_w, D, "norm weight"), float(eps),
+        h.data_ptr() if in_w is not None else 0, _code(h) if in_w is not None else 0, ldh,
+        _i32(rows, n_out, "rows") if rows is not None else 0, _stream()), "streams_step")
+
+
+def embed_streams(table: torch.Tensor, tokens: torch.Tensor, norm_w: Optional[torch.Tensor], eps: float,
+                  x: torch.Tensor, n_streams: int) -> None:
+    """x[t] = S copies of rms_norm(table[tokens[t]]) * norm_w (of the bare row without norm_w)."""
+    _gpu(table, tokens, norm_w, x)
+    T = tokens.numel()
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be a contiguous [vocab, width] matrix")
+    D = table.shape[1]
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.shape == (T, n_streams * D),
+          "embed_streams: x must be contiguous float32 [tokens, streams * width]")
+    L = _lib.load("plain")
+    _lib.check(L.apc_embed_streams(table.data_ptr(), _code(table), _i32(tokens, T, "tokens"),
+                                   _f32(norm_w, D, "norm weight"), float(eps), x.data_ptr(), T, int(n_streams), D,
+                                   _stream()), "embed_streams")
+
+
+def clamped_glu_mul(gate_up: torch.Tensor, out: torch.Tensor, alpha: float, limit: float) -> None:
+    _gpu(gate_up, out)
+    ldg, ldo = _rows(gate_up, "clamped_glu in"), _rows(out, "clamped_glu out")
+    T, F = out.shape
+    _need(gate_up.shape == (T, 2 * F), "clamped_glu: input must be [rows, 2*F] (gate columns, then up columns)")
+    L = _lib.load("plain")
+    for r0 in range(0, T, 32768):
+        n = min(32768, T - r0)
+        _lib.check(L.apc_clamped_glu(gate_up[r0:].data_ptr(), _code(gate_up), ldg, out[r0:].data_ptr(), _code(out),
+                                     ldo, n, F, float(alpha), float(limit), _stream()), "clamped_glu")
+
+
+def clamped_glu(h: torch.Tensor, w_gate_up, out: torch.Tensor, alpha: float, limit: float) -> None:
+    """out[t, f] = g * sigmoid(alpha g) * (u + 1), g = min(h . Wg[f], limit), u = clamp(h . Wu[f], -limit, limit);
+    w_gate_up is [Wg; Wu] of shape [2F, D], or the pair of their tiled forms."""
+    T, F = out.shape
+    if isinstance(w_gate_up, tuple):
+        from . import tuned
+        if tuned.clamped_glu_bf16(h, w_gate_up[0], w_gate_up[1], out, alpha, limit):
+            return
+        gu = torch.empty((T, 2 * F), dtype=torch.float32, device=h.device)
+        tuned.gemm_bf16(h, w_gate_up[0], gu[:, :F])
+        tuned.gemm_bf16(h, w_gate_up[1], gu[:, F:])
+    else:
+        gu = torch.empty((T, 2 * F), dtype=torch.float32, device=h.device)
+        gemm_plain(h, w_gate_up, gu)
+    clamped_glu_mul(gu, out, alpha, limit)
+
+
+def scale_(x: torch.Tensor, s: float) -> None:
+    _gpu(x)
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "scale_: contiguous float32")
+    L = _lib.load("plain")
+    _lib.check(L.apc_scale(x.data_ptr(), float(s), x.numel(), _stream()), "scale")

@@ -454,3 +454,15 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
             step.row_seg.data_ptr(), rows, int(window), sc, kw, n_parts, ws.data_ptr(), 0, stream),
             "attention_decode_bf16")
     return True
+
+
+def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens, block_table, step,
+                          mask: str, mask_size: int, sink: bool, scale: float) -> bool:
+    """Attention with a chunked or sliding mask and an optional sink on the MFMA kernels; False for sizes they do not
+    take (the caller then runs the plain kernel)."""
+    return False
+
+
+def clamped_glu_bf16(h, wg: PackedWeight, wu: PackedWeight, out, alpha: float, limit: float) -> bool:
+    """The clamped gated activation in the epilogue of the gate and up products; False where there is no kernel."""
+    return False

@@ -21,14 +21,15 @@ ARCHITECTURES: Registry = Registry("architecture")
 
 
 def architecture_of(config_json: Mapping[str, Any]) -> Architecture:
-    """By `architectures[0]`, then by `model_type`."""
+    """By `architectures[0]`, then by `architecture`, then by `model_type`."""
     names = list(config_json.get("architectures") or [])
-    candidates = names[:1] + ([config_json["model_type"]] if config_json.get("model_type") else [])
+    candidates = names[:1] + [config_json[k] for k in ("architecture", "model_type")
+                              if isinstance(config_json.get(k), str) and config_json[k]]
     for n in candidates:
         if n in ARCHITECTURES:
             return ARCHITECTURES.get(n)
     if not candidates:
-        raise ConfigError("config.json names no architecture (keys 'architectures' and 'model_type' are both absent)")
+        raise ConfigError("config.json names no architecture (keys 'architectures', 'architecture' and 'model_type' are all absent)")
     raise ConfigError(f"config.json names architecture {candidates!r}; known: {', '.join(ARCHITECTURES.names())}")
 
 
@@ -40,7 +41,7 @@ def describe_model(config_json: Mapping[str, Any]) -> Tuple[Architecture, Any, M
     return arch, cfg, spec
 
 
-from . import llama  # noqa: E402,F401  (registers itself)
+from . import llama, risizen  # noqa: E402,F401  (they register themselves)
 from .decoder import DecoderModel, load_model  # noqa: E402
 
 __all__ = ["ARCHITECTURES", "Architecture", "architecture_of", "describe_model", "DecoderModel", "load_model"]

@@ -26,6 +26,8 @@ class DecoderModel:
         self.final_norm = build_part(NORMS, spec.final_norm)
         self.head = build_part(HEADS, spec.head)
         self.rt: Optional[Runtime] = None
+        # called with (plan entry, residual) after every entry when set: a debugging aid (it is not part of a graph)
+        self.layer_tap = None
 
     # ---- weights -----------------------------------------------------------
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -55,6 +57,11 @@ class DecoderModel:
         else:
             self.head.bind(local(self.spec.head.weight_prefix, self.head), rt)
 
+    def _ones(self, n: int) -> torch.Tensor:
+        if getattr(self, "_ones_t", None) is None or self._ones_t.numel() != n:
+            self._ones_t = torch.ones(n, dtype=torch.float32, device=self.rt.device)
+        return self._ones_t
+
     # ---- cache needs, one per plan entry -------------------------------------
     def cache_needs(self) -> List[CacheNeed]:
         """What each plan entry needs of the cache manager: None (it borrows, or keeps nothing), one need (only the
@@ -62,7 +69,7 @@ class DecoderModel:
         role -> need (the arrangement gets a dict role -> view)."""
         needs: List[CacheNeed] = []
         for e in self.spec.plan:
-            asked = {} if e.cache_of is not None else self.blocks[e.block].cache_needs()
+            asked = self.blocks[e.block].cache_needs(borrows=e.cache_of is not None)
             needs.append(None if not asked else asked["mixer"] if list(asked) == ["mixer"] else asked)
         return needs
 
@@ -76,8 +83,10 @@ class DecoderModel:
 
     # The same in three pieces, for callers that record the step's launches in more than one graph.
     def embed(self, step) -> torch.Tensor:
-        """The float32 residual stream [rows, hidden] of the step's tokens."""
-        x = torch.empty((step.n_rows, self.spec.hidden_size), dtype=torch.float32, device=self.rt.device)
+        """The float32 residual stream [rows, hidden] of the step's tokens ([rows, streams * hidden] for a model
+        with several residual streams)."""
+        x = torch.empty((step.n_rows, self.spec.streams * self.spec.hidden_size), dtype=torch.float32,
+                        device=self.rt.device)
         self.embedding.forward(step.tokens, x)
         return x
 
@@ -88,6 +97,8 @@ class DecoderModel:
         for i in range(lo, hi):
             nxt = self.blocks[plan[i + 1].block].first_norm() if i + 1 < len(plan) else None
             left = self.blocks[plan[i].block].run(x, step, caches[i], pre=left, next_norm=nxt)
+            if self.layer_tap is not None:
+                self.layer_tap(i, x)
         return left
 
     def logits(self, x: torch.Tensor, step) -> Optional[torch.Tensor]:
@@ -96,7 +107,13 @@ class DecoderModel:
             return None
         rt = self.rt
         h = torch.empty((R, self.spec.hidden_size), dtype=rt.dtype, device=rt.device)
-        self.final_norm.forward(x, h, rows=step.logit_rows)
+        if self.spec.streams > 1:      # the streams are summed in front of the final norm
+            from ..kernels import ops
+            S = self.spec.streams
+            w, eps = self.final_norm.rms_params()
+            ops.streams_step(x, S, in_w=self._ones(S), norm_w=w, eps=eps, h=h, rows=step.logit_rows)
+        else:
+            self.final_norm.forward(x, h, rows=step.logit_rows)
         logits = torch.empty((R, self.spec.vocab_size), dtype=torch.float32, device=rt.device)
         self.head.forward(h, logits)
         return logits

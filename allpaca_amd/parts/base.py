@@ -29,6 +29,7 @@ FEED_FORWARDS: Registry = Registry("feed-forward")
 NORMS: Registry = Registry("norm")
 POSITION_ENCODINGS: Registry = Registry("position encoding")
 ARRANGEMENTS: Registry = Registry("block arrangement")
+CONNECTIONS: Registry = Registry("residual connection")
 EMBEDDINGS: Registry = Registry("embedding")
 HEADS: Registry = Registry("output head")
 
@@ -55,6 +56,21 @@ class PagedKV:
 
     def page_shape(self, page_tokens: int) -> Tuple[int, ...]:
         return (2, self.kv_heads, page_tokens, self.head_dim)
+
+
+@dataclass(frozen=True)
+class PagedKeysValues:
+    """Keys of `key_dim` and values of `value_dim` elements a head, of every position (or of the last `window`), in
+    pages of one row per kv head: first the page's keys [slot][key_dim], then its values [value_dim][slot]."""
+    kv_heads: int
+    key_dim: int
+    value_dim: int
+    window: Optional[int] = None
+    kind = "pages"
+    dtype = None
+
+    def page_shape(self, page_tokens: int) -> Tuple[int, ...]:
+        return (self.kv_heads, page_tokens * (self.key_dim + self.value_dim))
 
 
 @dataclass(frozen=True)
@@ -221,6 +237,12 @@ class Mixer(Part):
     # True if `forward_add` takes `emit=` (a `NormEmit` or None) for its product into the residual
     emits_next_norm = False
     def cache_need(self) -> CacheNeed:
+        """What the mixer keeps per request that a later plan entry may read in its place (`PlanEntry.cache_of`)."""
+        return None
+
+    def state_need(self) -> CacheNeed:
+        """What the mixer keeps per request for itself alone, whether or not it reads another entry's cache: the
+        arrangement gets it under the role "<role>.state"."""
         return None
 
     def forward(self, h: torch.Tensor, step, cache) -> torch.Tensor:

@@ -7,7 +7,7 @@ from typing import Dict, Mapping
 
 import torch
 
-from .base import ARRANGEMENTS, FEED_FORWARDS, MIXERS, NORMS, NormEmit, NormedInput, Part, build_part
+from .base import ARRANGEMENTS, CONNECTIONS, FEED_FORWARDS, MIXERS, NORMS, NormEmit, NormedInput, Part, build_part
 from .spec import BlockSpec
 
 
@@ -41,16 +41,18 @@ class Block:
     def mixer(self):
         return self.parts["mixer"]
 
-    def cache_needs(self) -> Dict[str, object]:
+    def cache_needs(self, borrows: bool = False) -> Dict[str, object]:
         """role -> what that part needs of the cache manager, for every part of the layer that keeps something per
         request (`cache_need()` answering other than None): attention heads beside recurrent heads are two roles with
-        a need each."""
+        a need each.  What a part keeps for itself alone (`state_need()`) stands under "<role>.state".  `borrows`: the
+        layer runs against another plan entry's cache, and only what its parts keep for themselves is asked for."""
         out = {}
         for role, part in self.parts.items():
-            ask = getattr(part, "cache_need", None)
-            need = ask() if callable(ask) else None
-            if need is not None:
-                out[role] = need
+            for name, key in (("cache_need", role), ("state_need", role + ".state")):
+                ask = getattr(part, name, None)
+                need = ask() if callable(ask) and not (borrows and name == "cache_need") else None
+                if need is not None:
+                    out[key] = need
         return out
 
     def native_desc(self):
@@ -110,3 +112,65 @@ class PreNorm:
         else:
             ffn.forward_add(h if ffn.takes_normed_input else h.tensor(), step, x)
         return emit if emit is not None and emit.filled else None
+
+
+class StreamsLeft:
+    """What a layer over residual streams leaves for the next one: the next layer's first input, already read from
+    the streams and normalised (the write of this layer's last output and that read are one pass over the row)."""
+
+    def __init__(self, connection, norm, h: torch.Tensor):
+        self.connection, self.norm, self.h = connection, norm, h
+
+
+class StreamsFirst:
+    """What a layer over residual streams shows the layer before it: the connection and the norm of its first read."""
+
+    def __init__(self, connection, norm):
+        self.connection, self.norm = connection, norm
+
+    def rms_params(self):       # to an arrangement that folds norms into products this is no norm it can fold
+        return None
+
+
+@ARRANGEMENTS.register("hyper_pre_norm")
+class HyperPreNorm:
+    """Over S residual streams x_1 .. x_S of a row (x is [rows, S * hidden] float32):
+       u = sum_a in1[a] x_a;  y = mixer(norm1(u));  x_b <- sum_a mix1[a][b] x_a + out1[b] y
+    and the same with the feed-forward and the second connection, if the layer has one."""
+    registries = {"mixer_norm": NORMS, "mixer": MIXERS, "mixer_link": CONNECTIONS,
+                  "ffn_norm": NORMS, "ffn": FEED_FORWARDS, "ffn_link": CONNECTIONS}
+    chains_norms = True
+
+    @staticmethod
+    def first_norm(parts):
+        return StreamsFirst(parts["mixer_link"], parts["mixer_norm"])
+
+    @staticmethod
+    def run(parts, x: torch.Tensor, step, cache, pre=None, next_norm=None):
+        mixer, link1, norm1 = parts["mixer"], parts["mixer_link"], parts["mixer_norm"]
+        ffn = parts.get("ffn")
+        rt = mixer.rt
+        T, D = x.shape[0], x.shape[1] // link1.S
+
+        def buffer():
+            return torch.empty((T, D), dtype=rt.dtype, device=x.device)
+
+        if isinstance(pre, StreamsLeft) and pre.connection is link1 and pre.norm is norm1:
+            h = pre.h
+        else:
+            h = buffer()
+            link1.read(x, norm1, h)
+        y = mixer.forward(h, step, cache)
+        last = link1
+        if ffn is not None:
+            link2, norm2 = parts["ffn_link"], parts["ffn_norm"]
+            h = buffer()
+            link1.write(x, y, then=link2, norm=norm2, h=h)
+            y = ffn.forward(h, step)
+            last = link2
+        if isinstance(next_norm, StreamsFirst) and next_norm.connection.S == last.S:
+            h = buffer()
+            last.write(x, y, then=next_norm.connection, norm=next_norm.norm, h=h)
+            return StreamsLeft(next_norm.connection, next_norm.norm, h)
+        last.write(x, y)
+        return None

@@ -33,25 +33,54 @@ class TokenEmbedding(Part):
         return {"kind": "token_table", "weight": self.weight} if type(self) is TokenEmbedding else None
 
 
+@EMBEDDINGS.register("token_table_norm")
+class NormedTokenEmbedding(Part):
+    """A token's row of the table through an RMS norm with a weight of its own (`norm_name`), written into every
+    residual stream of the row."""
+    graph_safe = True
+
+    def __init__(self, vocab_size: int, hidden_size: int, eps: float, streams: int = 1, table_name: str = "weight",
+                 norm_name: str = "norm"):
+        self.V, self.D, self.eps, self.S = int(vocab_size), int(hidden_size), float(eps), int(streams)
+        self.table_name, self.norm_name = table_name, norm_name
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {self.table_name: ParamSpec((self.V, self.D)), self.norm_name: ParamSpec((self.D,), store="float32")}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+        self.weight = to_device(tensors[self.table_name], rt)      # row-major: rows are read whole
+        self.norm_weight = to_device(tensors[self.norm_name], rt, torch.float32)
+
+    def forward(self, tokens: torch.Tensor, out: torch.Tensor) -> None:
+        ops.embed_streams(self.weight, tokens, self.norm_weight, self.eps, out, self.S)
+
+
 @HEADS.register("linear")
 class LinearHead(Part):
     """`tied`: the head uses the embedding matrix and owns no tensor."""
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False):
+    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False, scale: float = 1.0,
+                 name: str = "weight"):
         self.V, self.D, self.tied = int(vocab_size), int(hidden_size), bool(tied)
+        self.scale, self.name = float(scale), name     # logits = (h W^T) * scale
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {} if self.tied else {"weight": ParamSpec((self.V, self.D))}
+        return {} if self.tied else {self.name: ParamSpec((self.V, self.D))}
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime, shared: Optional[torch.Tensor] = None) -> None:
         self.rt = rt
-        self.weight = shared if self.tied else ops.prepare_matrix(to_device(tensors["weight"], rt), rt.dtype)
+        self.weight = shared if self.tied else ops.prepare_matrix(to_device(tensors[self.name], rt), rt.dtype)
         if self.weight is None:
             raise ValueError("a tied head needs the embedding matrix")
 
     def forward(self, h: torch.Tensor, out: torch.Tensor) -> None:
         ops.linear(h, self.weight, out)
+        if self.scale != 1.0:
+            ops.scale_(out, self.scale)
 
     def native_desc(self):
-        return {"kind": "linear", "weight": self.weight} if type(self) is LinearHead else None
+        if type(self) is not LinearHead or self.scale != 1.0:
+            return None
+        return {"kind": "linear", "weight": self.weight}

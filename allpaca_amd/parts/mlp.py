@@ -57,3 +57,38 @@ class SwiGLU(FeedForward):
         out = torch.zeros((h.shape[0], self.D), dtype=torch.float32, device=h.device)
         self.forward_add(h, step, out)
         return out
+
+
+@FEED_FORWARDS.register("clamped_glu")
+class ClampedGLU(FeedForward):
+    """g = min(h Wg^T, limit), u = clamp(h Wu^T, -limit, limit), a = g * sigmoid(alpha g) * (u + 1), out = a Wd^T,
+    no bias."""
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, alpha: float = 1.702,
+                 names: Mapping[str, str] | None = None):
+        self.D, self.F = int(hidden_size), int(intermediate_size)
+        self.limit, self.alpha = float(limit), float(alpha)
+        self.names = {"gate": "gate", "up": "up", "down": "down", **dict(names or {})}
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        n = self.names
+        return {n["gate"]: ParamSpec((self.F, self.D)), n["up"]: ParamSpec((self.F, self.D)),
+                n["down"]: ParamSpec((self.D, self.F))}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+        n = self.names
+        g, u = tensors[n["gate"]], tensors[n["up"]]
+        dt = g.dtype if g.dtype == u.dtype else torch.float32
+        wg, wu = ops.prepare_matrix(to_device(g, rt, dt), rt.dtype), ops.prepare_matrix(to_device(u, rt, dt), rt.dtype)
+        self.w_gate_up = torch.cat([wg, wu], dim=0).contiguous() if isinstance(wg, torch.Tensor) else (wg, wu)
+        self.w_down = ops.prepare_matrix(to_device(tensors[n["down"]], rt), rt.dtype)
+
+    def forward(self, h, step) -> torch.Tensor:
+        h = as_normed(h).tensor()
+        act = torch.empty((h.shape[0], self.F), dtype=self.rt.dtype, device=h.device)
+        ops.clamped_glu(h, self.w_gate_up, act, self.alpha, self.limit)
+        out = torch.empty((h.shape[0], self.D), dtype=torch.float32, device=h.device)
+        ops.linear(act, self.w_down, out)
+        return out

@@ -16,15 +16,15 @@ from .spec import ParamSpec
 class RMSNorm(Norm):
     graph_safe = True
 
-    def __init__(self, size: int, eps: float):
-        self.size, self.eps = int(size), float(eps)
+    def __init__(self, size: int, eps: float, name: str = "weight"):
+        self.size, self.eps, self.name = int(size), float(eps), name     # `name`: the weight's tensor name
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.size,), store="float32")}
+        return {self.name: ParamSpec((self.size,), store="float32")}
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
         self.rt = rt
-        self.weight = to_device(tensors["weight"], rt, torch.float32)
+        self.weight = to_device(tensors[self.name], rt, torch.float32)
 
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
         ops.rmsnorm_rows(x, self.weight, self.eps, out, rows)

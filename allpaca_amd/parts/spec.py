@@ -72,6 +72,10 @@ class ModelSpec:
     # axes of a token's position that the position encodings read: 1 (the place in the request), or more, and then a
     # step carries int32 [rows, axes] beside the places (`StepInfo.position_axes`, given per request in `Entry.positions`)
     position_axes: int = 1
+    # copies of the residual a row carries ([rows, streams * hidden_size] float32, all equal to the embedding's output
+    # at the start, summed in front of the final norm); arrangements that read and write them with weights of their
+    # own say how they are used
+    streams: int = 1
 
     def validate(self) -> None:
         for i, e in enumerate(self.plan):

@@ -80,11 +80,15 @@ def random_tensors(specs: Mapping[str, ParamSpec], seed: int, dtype: torch.dtype
             t = torch.ones(ps.shape, dtype=torch.float32, device=dev)
             if norm_std:
                 t += unit_normal(_tensor_seed(seed, name), count, dev).view(ps.shape) * float(norm_std)
+        elif init == "identity_plus_normal":
+            t = torch.eye(ps.shape[0], ps.shape[1], dtype=torch.float32, device=dev)
+            if norm_std:
+                t += unit_normal(_tensor_seed(seed, name), count, dev).view(ps.shape) * float(norm_std)
         elif init == "normal":
             t = unit_normal(_tensor_seed(seed, name), count, dev).view(ps.shape)
             t *= float(std)
         else:
-            raise ValueError(f"tensor {name!r}: init {init!r} is not 'normal', 'ones_plus_normal', 'zeros' or a number")
+            raise ValueError(f"tensor {name!r}: init {init!r} is not 'normal', 'ones_plus_normal', 'identity_plus_normal', 'zeros' or a number")
         out[name] = t.to(want)
     return out
 
