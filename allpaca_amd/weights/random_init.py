@@ -108,8 +108,9 @@ def write_model_folder(path: str, config_json: Mapping[str, Any], seed: int, dty
     the same values wherever)."""
     from ..models import DecoderModel, describe_model
     _, cfg, spec = describe_model(config_json)
-    specs = DecoderModel(spec).param_specs()
     overrides = dict(overrides or {})
+    # a tensor the model can do without is written only if the caller brings it
+    specs = {n: ps for n, ps in DecoderModel(spec).param_specs().items() if not ps.optional or n in overrides}
     for name, t in overrides.items():
         if name not in specs:
             raise KeyError(f"override {name!r} is not a tensor of this model")

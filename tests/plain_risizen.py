@@ -37,15 +37,18 @@ def short_conv(u: np.ndarray, w: np.ndarray, before: Optional[np.ndarray] = None
     return y
 
 
-def visible(i: int, j: int, chunk: Optional[int]) -> bool:
-    """Whether position i sees position j: causal, and inside the same chunk (counted from position 0)."""
+def visible(i: int, j: int, chunk: Optional[int], window: Optional[int] = None) -> bool:
+    """Whether position i sees position j: causal, inside the same chunk (counted from position 0), and among the
+    last `window` positions (the design itself has chunks only; the engine's kernel also takes a window)."""
     if j > i:
+        return False
+    if window is not None and i - j >= window:
         return False
     return chunk is None or (i // chunk) == (j // chunk)
 
 
 def sink_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, chunk: Optional[int],
-                   pos0: int = 0, sink: bool = True) -> np.ndarray:
+                   pos0: int = 0, sink: bool = True, window: Optional[int] = None) -> np.ndarray:
     """q [Tq, H, dk] at positions pos0 + (len(k) - Tq) ..., k [Tk, G, dk], v [Tk, G, dv] at positions pos0 ...
     Query head h reads key/value head h // (H / G).  p_j = exp(s_j) / (1 + sum_j exp(s_j)): the 1 is a sink with
     score 0 and no value.  Returns [Tq, H * dv]."""
@@ -55,7 +58,7 @@ def sink_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, ch
     first_q = pos0 + Tk - Tq
     for a in range(Tq):
         i = first_q + a
-        js = [j for j in range(Tk) if visible(i, pos0 + j, chunk)]
+        js = [j for j in range(Tk) if visible(i, pos0 + j, chunk, window)]
         for h in range(H):
             g = h // (H // G)
             s = (k[js, g] @ q[a, h]) * scale
