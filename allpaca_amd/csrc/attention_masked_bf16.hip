@@ -1,0 +1,540 @@
+// Attention with a mask of chunks or a sliding window, an optional sink, and keys and values of different sizes, in
+// bfloat16 on MFMA with float32 softmax.
+//
+//   the row at position p sees keys lo(p) .. p:  lo = 0 (causal), max(0, p - n + 1) (window of n), p - p % n (chunks of
+//   n positions counted from position 0);  s = (q . k) * scale;  weights exp(s) / (sink + sum exp(s)), sink = 1 (a key
+//   of score 0 without a value) or 0;  query head h reads kv head h / (H / G).
+//
+// Pages: one row per kv head, first the page's keys [slot][dk], then its values [dv][slot]; a page is
+// G * P * (dk + dv) elements.
+//
+//   prompt portions  a block of 4 waves takes up to 64 consecutive rows of one request x one head, 16 rows a wave on
+//                    v_mfma_f32_16x16x32_bf16; keys and values in tiles of 64 through LDS; online softmax whose running
+//                    maximum starts at the sink's score.  The products are transposed (S^T = K Q^T, O^T = V^T P^T), as
+//                    in attention_bf16.hip, so a row's maximum and sum are registers of 4 lanes.
+//   decoded rows     one row x one kv head x one range of its keys a block: a thread takes a key and forms its score with
+//                    every query head of the group (keys are read once a group), the block's 256 weights a head go
+//                    through LDS, a thread then owns one value element and adds up its keys' values page by page (a
+//                    page's slots of an element lie together).  A second kernel adds the ranges and the sink.
+#include "mfma.h"
+#include <math.h>
+
+namespace {
+
+constexpr int KT = 64;
+constexpr int QT = 64;
+constexpr int KPAD = 8;
+constexpr float LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ int first_seen(int pos, int mask, int size) {
+  if (mask == 1) return pos - size + 1 > 0 ? pos - size + 1 : 0;
+  if (mask == 2) return pos - pos % size;
+  return 0;
+}
+__device__ __forceinline__ float row4_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16, WAVE));
+  return fmaxf(v, __shfl_xor(v, 32, WAVE));
+}
+__device__ __forceinline__ float row4_sum(float v) {
+  v += __shfl_xor(v, 16, WAVE);
+  return v + __shfl_xor(v, 32, WAVE);
+}
+// all but the positions lo <= p < hi of a value operand's 8 are cleared (what lies there may be anything, and
+// 0 x NaN is NaN)
+__device__ __forceinline__ void keep_positions(Frag& v, int lo, int hi) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const uint32_t a = (2 * w >= lo && 2 * w < hi) ? 0x0000ffffu : 0u;
+    const uint32_t b = (2 * w + 1 >= lo && 2 * w + 1 < hi) ? 0xffff0000u : 0u;
+    v.w[w] &= a | b;
+  }
+}
+__device__ __forceinline__ float exp2_neg(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ------------------------------------------------------------------------------------------ prompt portions
+template <int DKP, int DVP>  // key and value sizes rounded up to a multiple of 32
+__global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
+    const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, int H, int G, int dk, int dv,
+    const bf16_t* __restrict__ cache, int P, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
+    const int* __restrict__ tile_rows, int n_tiles, int mask, int mask_size, int sink, float scale) {
+  constexpr int KROW = DKP + (DKP % 128 == 0 ? 72 : DKP % 128 == 64 ? 8 : DKP % 128 == 32 ? 40 : 104);
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KROW];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[DVP * (KT + KPAD)];
+  __shared__ __attribute__((aligned(16))) bf16_t Ps[4 * 16 * (KT + KPAD)];
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  const int li = lane % 16, lc = lane / 16;
+  // all heads that read one kv head run on one XCD (blocks go to the 8 XCDs in turn), tiles from the last to the first
+  int tile, h;
+  {
+    const int id = blockIdx.x, per = H / G;
+    if (G % 8 == 0) {
+      const int xcd = id % 8, slot = id / 8;
+      const int lh = slot / n_tiles;
+      tile = n_tiles - 1 - slot % n_tiles;
+      h = (xcd + 8 * (lh / per)) * per + lh % per;
+    } else {
+      tile = n_tiles - 1 - id % n_tiles;
+      h = id / n_tiles;
+    }
+  }
+  // the step's tiles have up to 2 QT rows; this kernel takes them in halves (n_tiles counts halves)
+  const int nrows = min(tile_rows[tile / 2] - (tile % 2) * QT, QT);
+  if (nrows <= 0) return;
+  const int row0 = tile_row0[tile / 2] + (tile % 2) * QT;
+  const int g = h / (H / G);
+  const int pos0 = positions[row0];
+  const int* bt = block_table + (size_t)row_seg[row0] * max_blocks;
+  const int last = pos0 + nrows - 1;
+  const int first = first_seen(pos0, mask, mask_size);   // the smallest of the rows' first keys
+  const size_t page_stride = (size_t)G * P * (dk + dv);
+  const int dchunks = dk / 8;
+
+  for (int idx = tid; idx < KT * KROW; idx += 256) Ks[idx] = 0;
+  for (int idx = tid; idx < DVP * (KT + KPAD); idx += 256) Vs[idx] = 0;
+
+  const int my_row = wave * 16 + li;
+  Frag qf[DKP / 32];
+  {
+    const bf16_t* qrow = q + (size_t)(row0 + min(my_row, nrows - 1)) * ldq + (size_t)h * dk;
+#pragma unroll
+    for (int ks = 0; ks < DKP / 32; ++ks) {
+      const int e = ks * 32 + lc * 8;
+      qf[ks] = (my_row < nrows && e < dk) ? load_frag(qrow + e) : zero_frag();
+    }
+  }
+  const int my_pos = pos0 + my_row;
+  const int my_lo = first_seen(my_pos, mask, mask_size);
+  const int wave_hi = pos0 + wave * 16;                        // smallest position of the wave's rows
+  const int wave_lo = first_seen(wave_hi + 15, mask, mask_size);  // largest first key of the wave's rows
+  const float sc2 = scale * LOG2E;
+  floatx4 o[DVP / 16];
+#pragma unroll
+  for (int dt = 0; dt < DVP / 16; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = sink ? 0.f : -INFINITY, l_run = sink ? 1.f : 0.f;   // the sink is the row's first "key"
+  bf16_t* pw = Ps + wave * 16 * (KT + KPAD) + li * (KT + KPAD);
+  const bf16_t* krd = Ks + li * KROW + lc * 8;
+  const bf16_t* vrd = Vs + li * (KT + KPAD) + lc * 8;
+
+  // A tile is 8 groups of 8 consecutive keys, a group lies in one page; the 32 threads of group tid / 32 copy its keys
+  // (8 x dk elements, consecutive in the page) and its values (dv rows of 8 slots).
+  constexpr int KP = DKP / 32, VP = DVP / 32;
+  const int grp = tid / 32, gl = tid % 32;
+  const int last_group = (last / 8) * 8;
+  int k_ldst[KP], v_ldst[VP];
+  bool k_on[KP], v_on[VP];
+#pragma unroll
+  for (int j = 0; j < KP; ++j) {
+    const int idx = gl + 32 * j;
+    k_on[j] = idx < dk;
+    const int key = k_on[j] ? idx / dchunks : 0, ch = k_on[j] ? idx % dchunks : 0;
+    k_ldst[j] = (grp * 8 + key) * KROW + ch * 8;
+  }
+#pragma unroll
+  for (int j = 0; j < VP; ++j) {
+    const int idx = gl + 32 * j;
+    v_on[j] = idx < dv;
+    v_ldst[j] = (v_on[j] ? idx : 0) * (KT + KPAD) + grp * 8;
+  }
+  const bf16_t* k_head = cache + (size_t)g * P * (dk + dv);
+  const bf16_t* v_head = k_head + (size_t)P * dk;
+  int page_next = 0;
+  auto lookup_tile = [&](int t0) { page_next = bt[min(t0 + grp * 8, last_group) / P]; };
+  Frag kreg[KP], vreg[VP];
+  int v_lo = 0, v_hi = 8;
+  auto load_tile = [&](int t0) {
+    const int tg = min(t0 + grp * 8, last_group), slot0 = tg % P;
+    v_lo = first - tg;
+    v_hi = last - tg + 1;
+    const bf16_t* kp = k_head + (size_t)page_next * page_stride + (size_t)slot0 * dk;
+    const bf16_t* vp = v_head + (size_t)page_next * page_stride + slot0;
+#pragma unroll
+    for (int j = 0; j < KP; ++j) kreg[j] = load_frag(kp + (k_on[j] ? gl + 32 * j : 0) * 8);
+#pragma unroll
+    for (int j = 0; j < VP; ++j) vreg[j] = load_frag(vp + (size_t)(v_on[j] ? gl + 32 * j : 0) * P);
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < KP; ++j)
+      if (k_on[j]) *reinterpret_cast<Frag*>(Ks + k_ldst[j]) = kreg[j];
+#pragma unroll
+    for (int j = 0; j < VP; ++j) {
+      if (v_on[j]) {
+        if (v_lo > 0 || v_hi < 8) keep_positions(vreg[j], v_lo, v_hi);
+        *reinterpret_cast<Frag*>(Vs + v_ldst[j]) = vreg[j];
+      }
+    }
+  };
+
+  const int t_begin = (first / KT) * KT;
+  lookup_tile(t_begin);
+  load_tile(t_begin);
+  lookup_tile(t_begin + KT);
+  __syncthreads();
+  store_tile();
+  __syncthreads();
+  for (int t0 = t_begin; t0 <= last; t0 += KT) {
+    load_tile(t0 + KT);
+    lookup_tile(t0 + 2 * KT);
+
+    floatx4 s[KT / 16];
+#pragma unroll
+    for (int nt = 0; nt < KT / 16; ++nt) {
+      s[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < DKP / 32; ++ks) {
+        const Frag kf = *reinterpret_cast<const Frag*>(krd + nt * 16 * KROW + ks * 32);
+        s[nt] = mfma16(kf, qf[ks], s[nt]);
+      }
+    }
+    float mx = -INFINITY;
+    if (t0 >= wave_lo && t0 + KT - 1 <= wave_hi) {
+#pragma unroll
+      for (int nt = 0; nt < KT / 16; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[nt][r]);
+    } else {
+#pragma unroll
+      for (int nt = 0; nt < KT / 16; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int t = t0 + nt * 16 + lc * 4 + r;
+          const float v = (t >= my_lo && t <= my_pos) ? s[nt][r] : -INFINITY;
+          s[nt][r] = v;
+          mx = fmaxf(mx, v);
+        }
+    }
+    mx = row4_max(mx) * sc2;
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2_neg(m_run - m_safe);
+    float sum = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < KT / 16; ++nt) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s[nt][r] = exp2_neg(fmaf(s[nt][r], sc2, -m_safe));
+        sum += s[nt][r];
+      }
+      uint2 pk;
+      pk.x = pack_bf16x2(s[nt][0], s[nt][1]);
+      pk.y = pack_bf16x2(s[nt][2], s[nt][3]);
+      *reinterpret_cast<uint2*>(pw + nt * 16 + lc * 4) = pk;
+    }
+    l_run = l_run * alpha + row4_sum(sum);
+    m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < DVP / 16; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+    }
+    wave_lds_order();
+#pragma unroll
+    for (int kstep = 0; kstep < KT / 32; ++kstep) {
+      const Frag pf = *reinterpret_cast<const Frag*>(pw + kstep * 32 + lc * 8);
+#pragma unroll
+      for (int dt = 0; dt < DVP / 16; ++dt) {
+        const Frag vf = *reinterpret_cast<const Frag*>(vrd + dt * 16 * (KT + KPAD) + kstep * 32);
+        o[dt] = mfma16(vf, pf, o[dt]);
+      }
+    }
+    __syncthreads();
+    store_tile();
+    __syncthreads();
+  }
+  if (my_row < nrows) {
+    const float inv = 1.0f / l_run;
+    bf16_t* orow = out + (size_t)(row0 + my_row) * ldo + (size_t)h * dv;
+#pragma unroll
+    for (int dt = 0; dt < DVP / 16; ++dt) {
+      const int e = dt * 16 + lc * 4;
+      if (e < dv) {
+        uint2 pk;
+        pk.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
+        pk.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+        *reinterpret_cast<uint2*>(orow + e) = pk;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------ decoded rows
+constexpr int DT = 256;       // keys of a pass: one a thread
+constexpr int DMAX = 256;     // largest key and value size
+
+// grid: rows x G x n_splits.  Split s of a row takes the keys at positions a0 + s * kps .. a0 + (s + 1) * kps - 1 that
+// the row sees, a0 being the row's first key rounded down to a multiple of DT (kps is a multiple of DT, pages are
+// powers of two up to DT: a pass starts at a page's first slot).  It leaves, per query head of the group, the maximum
+// score m, sum exp(s - m) and sum exp(s - m) v of its keys in `parts` [row][head][split][2 + dv].
+template <int HG>  // query heads of a kv head, rounded up to a power of two
+__global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
+    const bf16_t* __restrict__ q, int ldq, int H, int G, int dk, int dv, const bf16_t* __restrict__ cache, int P,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ positions,
+    const int* __restrict__ row_seg, const int* __restrict__ rows, int mask, int mask_size, float scale, int n_splits,
+    int kps, float* __restrict__ parts) {
+  __shared__ __attribute__((aligned(16))) float qs[HG * DMAX];
+  __shared__ __attribute__((aligned(16))) float ps[HG * DT];
+  __shared__ float red[2][HG][DT / WAVE];
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  const int split = blockIdx.x % n_splits, g = (blockIdx.x / n_splits) % G, ri = blockIdx.x / (n_splits * G);
+  const int r = rows ? rows[ri] : ri;
+  const int per = H / G;                        // query heads of this kv head (<= HG)
+  const int pos = positions[r];
+  const int first = first_seen(pos, mask, mask_size);
+  const int a0 = (first / DT) * DT;
+  const int* bt = block_table + (size_t)row_seg[r] * max_blocks;
+  const size_t page_stride = (size_t)G * P * (dk + dv);
+  const bf16_t* head = cache + (size_t)g * P * (dk + dv);
+
+  for (int idx = tid; idx < per * dk; idx += DT) {
+    const int j = idx / dk, i = idx % dk;
+    qs[j * DMAX + i] = bf16_to_float(q[(size_t)r * ldq + (size_t)(g * per + j) * dk + i]) * scale;
+  }
+  // the thread's value element and its share of a pass's pages
+  int dvt = 1;
+  while (dvt < dv) dvt <<= 1;
+  const int e = tid % dvt, sl = tid / dvt, nsl = DT / dvt;
+  float m_run[HG], l_run[HG], o[HG];
+#pragma unroll
+  for (int j = 0; j < HG; ++j) { m_run[j] = -INFINITY; l_run[j] = 0.f; o[j] = 0.f; }
+  __syncthreads();
+
+  const int lo_t = a0 + split * kps;
+  const int hi_t = min(lo_t + kps, pos + 1);
+  for (int t0 = lo_t; t0 < hi_t; t0 += DT) {
+    if (t0 + DT <= first) continue;             // (only the first pass of the first split can lie in front)
+    // scores of key t0 + tid with every head of the group
+    const int t = t0 + tid;
+    const bool valid = t >= first && t <= pos;
+    float s[HG];
+#pragma unroll
+    for (int j = 0; j < HG; ++j) s[j] = 0.f;
+    if (valid) {
+      const bf16_t* kp = head + (size_t)bt[t / P] * page_stride + (size_t)(t % P) * dk;
+      for (int c = 0; c < dk; c += 8) {
+        const Frag kf = load_frag(kp + c);
+        float kv[8];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          kv[2 * w] = __uint_as_float(kf.w[w] << 16);
+          kv[2 * w + 1] = __uint_as_float(kf.w[w] & 0xffff0000u);
+        }
+#pragma unroll
+        for (int j = 0; j < HG; ++j) {
+          if (j < per) {
+            const float4 qa = *reinterpret_cast<const float4*>(qs + j * DMAX + c);
+            const float4 qb = *reinterpret_cast<const float4*>(qs + j * DMAX + c + 4);
+            float a = s[j];
+            a = fmaf(qa.x, kv[0], a); a = fmaf(qa.y, kv[1], a); a = fmaf(qa.z, kv[2], a); a = fmaf(qa.w, kv[3], a);
+            a = fmaf(qb.x, kv[4], a); a = fmaf(qb.y, kv[5], a); a = fmaf(qb.z, kv[6], a); a = fmaf(qb.w, kv[7], a);
+            s[j] = a;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < HG; ++j) {
+      if (j < per) {
+        const float v = wave_max(valid ? s[j] : -INFINITY);
+        if (lane == 0) red[0][j][wave] = v;
+      }
+    }
+    __syncthreads();                            // (also: the pass before is done with ps)
+    float alpha[HG];
+#pragma unroll
+    for (int j = 0; j < HG; ++j) {
+      alpha[j] = 1.f;
+      if (j < per) {
+        float m_new = m_run[j];
+#pragma unroll
+        for (int w = 0; w < DT / WAVE; ++w) m_new = fmaxf(m_new, red[0][j][w]);   // finite: the pass holds a key the row sees
+        alpha[j] = __expf(m_run[j] - m_new);
+        m_run[j] = m_new;
+        const float p = valid ? __expf(s[j] - m_new) : 0.f;
+        ps[j * DT + tid] = p;
+        const float sum = wave_sum(p);
+        if (lane == 0) red[1][j][wave] = sum;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < HG; ++j) {
+      if (j < per) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < DT / WAVE; ++w) sum += red[1][j][w];
+        l_run[j] = l_run[j] * alpha[j] + sum;
+        o[j] *= alpha[j];
+      }
+    }
+    // values: element e of the pages sl, sl + nsl, ... of the pass
+    if (e < dv) {
+      for (int tp = t0 + sl * P; tp < t0 + DT; tp += nsl * P) {
+        if (tp > pos || tp + P <= first) continue;
+        const bf16_t* vp = head + (size_t)bt[tp / P] * page_stride + (size_t)P * dk + (size_t)e * P;
+        for (int c = 0; c < P; c += 8) {
+          const Frag vf = load_frag(vp + c);
+          float vv[8];
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            vv[2 * w] = __uint_as_float(vf.w[w] << 16);
+            vv[2 * w + 1] = __uint_as_float(vf.w[w] & 0xffff0000u);
+          }
+#pragma unroll
+          for (int i = 0; i < 8; ++i)             // slots the row does not see may hold anything
+            if (tp + c + i < first || tp + c + i > pos) vv[i] = 0.f;
+          const int k0 = tp - t0 + c;
+#pragma unroll
+          for (int j = 0; j < HG; ++j) {
+            if (j < per) {
+              const float4 pa = *reinterpret_cast<const float4*>(ps + j * DT + k0);
+              const float4 pb = *reinterpret_cast<const float4*>(ps + j * DT + k0 + 4);
+              float a = o[j];
+              a = fmaf(pa.x, vv[0], a); a = fmaf(pa.y, vv[1], a); a = fmaf(pa.z, vv[2], a); a = fmaf(pa.w, vv[3], a);
+              a = fmaf(pb.x, vv[4], a); a = fmaf(pb.y, vv[5], a); a = fmaf(pb.z, vv[6], a); a = fmaf(pb.w, vv[7], a);
+              o[j] = a;
+            }
+          }
+        }
+      }
+    }
+  }
+  // the threads that share an element add up through LDS (qs is free now: every pass is behind a barrier)
+  __syncthreads();
+  float* acc = qs;                               // [HG][DT]: DT <= DMAX
+#pragma unroll
+  for (int j = 0; j < HG; ++j)
+    if (j < per) acc[j * DMAX + tid] = o[j];
+  __syncthreads();
+  if (sl == 0 && e < dv) {
+#pragma unroll
+    for (int j = 0; j < HG; ++j) {
+      if (j < per) {
+        float sum = 0.f;
+        for (int k = 0; k < nsl; ++k) sum += acc[j * DMAX + k * dvt + e];
+        parts[(((size_t)ri * H + g * per + j) * n_splits + split) * (dv + 2) + 2 + e] = sum;
+      }
+    }
+  }
+  if (tid < per) {
+    float* p = parts + (((size_t)ri * H + g * per + tid) * n_splits + split) * (dv + 2);
+    float m = -INFINITY, l = 0.f;
+#pragma unroll
+    for (int j = 0; j < HG; ++j)
+      if (j == tid) { m = m_run[j]; l = l_run[j]; }
+    p[0] = m;
+    p[1] = l;
+  }
+}
+
+// out[row][head] = sum_s e^(m_s - M) o_s / (sink e^(-M) + sum_s e^(m_s - M) l_s),  M = max(m_s, 0 with a sink)
+__global__ __launch_bounds__(64) void attn_masked_merge_kernel(const float* __restrict__ parts, int n_splits, int H,
+                                                               int dv, const int* __restrict__ rows, int sink,
+                                                               bf16_t* __restrict__ out, int ldo) {
+  const int ri = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int r = rows ? rows[ri] : ri;
+  const float* p = parts + ((size_t)ri * H + h) * n_splits * (dv + 2);
+  float M = sink ? 0.f : -INFINITY;
+  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, p[(size_t)s * (dv + 2)]);
+  float L = sink ? __expf(-M) : 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float m = p[(size_t)s * (dv + 2)];
+    if (m != -INFINITY) L += __expf(m - M) * p[(size_t)s * (dv + 2) + 1];
+  }
+  const float inv = 1.0f / L;
+  for (int e = lane; e < dv; e += WAVE) {
+    float a = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float m = p[(size_t)s * (dv + 2)];
+      if (m != -INFINITY) a = fmaf(__expf(m - M), p[(size_t)s * (dv + 2) + 2 + e], a);
+    }
+    out[(size_t)r * ldo + (size_t)h * dv + e] = float_to_bf16(a * inv);
+  }
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+int check_sizes(const void* q, int ldq, const void* out, int ldo, const void* cache, int H, int G, int dk, int dv, int P,
+                int mask, int mask_size, float scale) {
+  if (H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || P <= 0 || mask < 0 || mask > 2 || (mask && mask_size <= 0))
+    return APC_ERR_BAD_ARG;
+  if (dk % 8 || dv % 4 || dk > DMAX || dv > DMAX || P % 8 || ldq % 8 || ldo % 4 || !aligned16(q) || !aligned16(cache) ||
+      ((uintptr_t)out & 7u) || !(scale > 0.f))
+    return APC_ERR_UNSUPPORTED;
+  return 0;
+}
+
+}  // namespace
+
+// 1 if the kernels take these sizes, else 0 (the caller then runs the plain kernel)
+APC_EXPORT int apc_attention_masked_takes(int H, int G, int dk, int dv, int page_tokens) {
+  if (H <= 0 || G <= 0 || H % G || H / G > 16) return 0;
+  if (dk % 8 || dv % 8 || dk > DMAX || dv > DMAX) return 0;
+  if (page_tokens < 8 || page_tokens > DT || (page_tokens & (page_tokens - 1))) return 0;
+  return 1;
+}
+
+APC_EXPORT int apc_attention_masked_prefill_bf16(const void* q, int ldq, void* out, int ldo, int H, int G, int dk,
+                                                 int dv, const void* cache, int page_tokens, const int* block_table,
+                                                 int max_blocks, const int* positions, const int* row_seg,
+                                                 const int* tile_row0, const int* tile_rows, int n_tiles, int mask,
+                                                 int mask_size, int sink, float scale, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale);
+  if (e) return e;
+  n_tiles *= 2;  // halves
+  if (max_blocks <= 0 || (long)n_tiles * H > 0x7fffffffL) return APC_ERR_BAD_ARG;
+  dim3 grid(n_tiles * H), block(256);
+#define MP_LAUNCH(DK_, DV_)                                                                                         \
+  hipLaunchKernelGGL((attn_masked_prefill_kernel<DK_, DV_>), grid, block, 0, stream, (const bf16_t*)q, ldq,          \
+                     (bf16_t*)out, ldo, H, G, dk, dv, (const bf16_t*)cache, page_tokens, block_table, max_blocks,    \
+                     positions, row_seg, tile_row0, tile_rows, n_tiles, mask, mask_size, sink, scale)
+#define MP_VALUES(DK_)                       \
+  do {                                       \
+    if (dv <= 64) MP_LAUNCH(DK_, 64);        \
+    else if (dv <= 128) MP_LAUNCH(DK_, 128); \
+    else MP_LAUNCH(DK_, 256);                \
+  } while (0)
+  if (dk <= 64) MP_VALUES(64);
+  else if (dk <= 128) MP_VALUES(128);
+  else MP_VALUES(256);
+#undef MP_VALUES
+#undef MP_LAUNCH
+  APC_LAUNCH_CHECK();
+  return 0;
+}
+
+// `rows`: the step's rows that are decoded ones (nullptr: all n_rows rows); `keys_per_split`: a multiple of 256;
+// `parts`: room for n_rows * H * n_splits * (dv + 2) floats.
+APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* out, int ldo, int n_rows, int H, int G,
+                                                int dk, int dv, const void* cache, int page_tokens,
+                                                const int* block_table, int max_blocks, const int* positions,
+                                                const int* row_seg, const int* rows, int mask, int mask_size, int sink,
+                                                float scale, int n_splits, int keys_per_split, float* parts,
+                                                hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale);
+  if (e) return e;
+  if (!apc_attention_masked_takes(H, G, dk, dv, page_tokens)) return APC_ERR_UNSUPPORTED;
+  if (n_splits <= 0 || keys_per_split <= 0 || keys_per_split % DT || !parts || max_blocks <= 0 ||
+      (long)n_rows * G * n_splits > 0x7fffffffL || H > 65535)
+    return APC_ERR_BAD_ARG;
+  dim3 grid(n_rows * G * n_splits), block(DT);
+  const int per = H / G;
+#define MD_LAUNCH(HG_)                                                                                              \
+  hipLaunchKernelGGL((attn_masked_decode_kernel<HG_>), grid, block, 0, stream, (const bf16_t*)q, ldq, H, G, dk, dv, \
+                     (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg, rows, mask,     \
+                     mask_size, scale, n_splits, keys_per_split, parts)
+  if (per <= 1) MD_LAUNCH(1);
+  else if (per <= 2) MD_LAUNCH(2);
+  else if (per <= 4) MD_LAUNCH(4);
+  else if (per <= 8) MD_LAUNCH(8);
+  else MD_LAUNCH(16);
+#undef MD_LAUNCH
+  APC_LAUNCH_CHECK();
+  hipLaunchKernelGGL(attn_masked_merge_kernel, dim3(n_rows, H), dim3(64), 0, stream, parts, n_splits, H, dv, rows, sink,
+                     (bf16_t*)out, ldo);
+  APC_LAUNCH_CHECK();
+  return 0;
+}

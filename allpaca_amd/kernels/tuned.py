@@ -456,11 +456,49 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
     return True
 
 
+MASKED_DECODE_BLOCKS = 1024   # blocks the decoded rows' key ranges are cut for (4 a compute unit)
+
+
 def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens, block_table, step,
                           mask: str, mask_size: int, sink: bool, scale: float) -> bool:
-    """Attention with a chunked or sliding mask and an optional sink on the MFMA kernels; False for sizes they do not
-    take (the caller then runs the plain kernel)."""
-    return False
+    """Attention with a chunked or sliding mask and an optional sink on the MFMA kernels: segments of several rows on
+    the tiled kernel, single rows on the kernel that cuts a row's keys into ranges.  False (nothing done) for sizes
+    they do not take; the caller then runs the plain kernel."""
+    _ops._gpu(q, out, cache, block_table)
+    ldq, ldo = _ops._rows(q, "attention q"), _ops._rows(out, "attention out")
+    T = q.shape[0]
+    L = _lib.load("tuned")
+    if (not scale > 0 or ldq % 8 or ldo % 4 or not _aligned(q, cache) or out.data_ptr() % 8
+            or q.dtype != torch.bfloat16 or cache.dtype != torch.bfloat16 or out.dtype != torch.bfloat16
+            or not L.apc_attention_masked_takes(n_heads, n_kv_heads, key_dim, value_dim, page_tokens)):
+        return False
+    _ops._need(q.shape[1] == n_heads * key_dim, "attention: q must be [rows, heads * key_dim]")
+    _ops._need(out.shape == (T, n_heads * value_dim), "attention out must be [rows, heads * value_dim]")
+    _ops._split_pages(cache, n_kv_heads, key_dim, value_dim, page_tokens)
+    _ops._need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+               "block table must be contiguous int32 [segments, blocks]")
+    _ops._need(step.positions.numel() >= T and step.row_seg.numel() >= T, "step rows differ from q rows")
+    code, stream = _ops.MASKS[mask], _ops._stream()
+    if step.n_tiles:
+        _lib.check(L.apc_attention_masked_prefill_bf16(
+            q.data_ptr(), ldq, out.data_ptr(), ldo, n_heads, n_kv_heads, key_dim, value_dim, cache.data_ptr(),
+            page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
+            step.row_seg.data_ptr(), step.tile_row0.data_ptr(), step.tile_rows.data_ptr(), step.n_tiles, code,
+            int(mask_size), 1 if sink else 0, float(scale), stream), "attention_masked_prefill_bf16")
+    if step.n_decode_rows:
+        n = step.n_decode_rows
+        keys = min(step.max_decode_context, mask_size) if code else step.max_decode_context
+        passes = -(-(keys + 255) // 256)        # a row's first pass starts at a multiple of 256 at or below its first key
+        splits = max(1, min(passes, MASKED_DECODE_BLOCKS // max(1, n * n_kv_heads)))
+        kps = -(-passes // splits) * 256
+        parts = torch.empty(n * n_heads * splits * (value_dim + 2), dtype=torch.float32, device=q.device)
+        _lib.check(L.apc_attention_masked_decode_bf16(
+            q.data_ptr(), ldq, out.data_ptr(), ldo, n, n_heads, n_kv_heads, key_dim, value_dim, cache.data_ptr(),
+            page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
+            step.row_seg.data_ptr(), step.decode_rows.data_ptr() if step.decode_rows is not None else 0, code,
+            int(mask_size), 1 if sink else 0, float(scale), splits, kps, parts.data_ptr(), stream),
+            "attention_masked_decode_bf16")
+    return True
 
 
 def clamped_glu_bf16(h, wg: PackedWeight, wu: PackedWeight, out, alpha: float, limit: float) -> bool:

@@ -127,7 +127,12 @@ def test_masked_attention_against_the_plain_one(mask, size, sink, dtype):
     qs = [R.unit_rms(rng.normal(size=(n, H, dk)), 1e-6) * 1.5 for n in rows]
     q = torch.as_tensor(np.concatenate(qs).reshape(T, H * dk), dtype=torch.float32).to(tdt).to(DEV)
     out = torch.empty((T, H * dv), dtype=tdt, device=DEV)
-    ops.masked_attention(q, out, H, G, dk, dv, cache, P_, step.block_tables[0], step, mask, size, sink, scale)
+    if dtype == "bfloat16":       # these sizes are ones the matrix-core kernels take: they must not pass them on
+        from allpaca_amd.kernels import tuned
+        assert tuned.masked_attention_bf16(q, out, H, G, dk, dv, cache, P_, step.block_tables[0], step, mask, size,
+                                           sink, scale)
+    else:
+        ops.masked_attention(q, out, H, G, dk, dv, cache, P_, step.block_tables[0], step, mask, size, sink, scale)
     want = []
     for k, v, qq in zip(ks, vs, qs):
         if dtype == "bfloat16":
@@ -143,7 +148,8 @@ def test_masked_attention_against_the_plain_one(mask, size, sink, dtype):
     ("window", 33, 400, 367, False), ("causal", 0, 900, 0, True), ("causal", 0, 900, 15, True),
     ("causal", 0, 900, 16, True)])
 @pytest.mark.parametrize("rows", [1, 70])
-def test_one_key_stands_out(mask, size, pos, key, seen, rows):
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_key_stands_out(mask, size, pos, key, seen, rows, dtype):
     """The last row's query points at one key with a large score: if the mask lets the row see it, the output is that
     key's value (a far key among hundreds, at a page's border, just inside a chunk or window); if not, it is not."""
     from allpaca_amd.kernels import ops
@@ -154,16 +160,17 @@ def test_one_key_stands_out(mask, size, pos, key, seen, rows):
     v = rng.normal(size=(L, G, dv))
     v[key] = 100.0 + np.arange(dv)
     table = [int(p) for p in rng.permutation(np.arange(1, -(-L // P_) + 1))]
-    cache = fill_pages(k, v, P_, table, torch.float32)
+    tdt = DTYPES[dtype]
+    cache = fill_pages(k, v, P_, table, tdt)
     n = min(rows, L)
     step = make_step([(L - n, n)], P_, [table], [0])
     qn = rng.normal(size=(n, H, dk))
     qn[-1, :] = k[key, 0] * 4.0                                 # score 4 * dk * scale = 32 against |others| of about 2
-    q = dev(qn.reshape(n, H * dk))
-    out = torch.empty((n, H * dv), dtype=torch.float32, device=DEV)
+    q = dev(qn.reshape(n, H * dk), tdt)
+    out = torch.empty((n, H * dv), dtype=tdt, device=DEV)
     ops.masked_attention(q, out, H, G, dk, dv, cache, P_, step.block_tables[0], step, mask, size, True, 0.5)
-    last = out[-1].cpu().numpy().reshape(H, dv)
-    hit = np.allclose(last, 100.0 + np.arange(dv), atol=0.5)     # (hundreds of other keys keep a sliver)
+    last = out[-1].float().cpu().numpy().reshape(H, dv)
+    hit = np.allclose(last, 100.0 + np.arange(dv), atol=0.5 if dtype == "float32" else 1.5)     # (hundreds of other keys keep a sliver)
     assert hit == seen, (last[0, :3], seen)
 
 
@@ -251,11 +258,12 @@ def run_cut(runner, toks, cuts, seq="s"):
 
 
 @pytest.mark.parametrize("name", ["RA", "RB", "RC", "RD"])
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_whole_prompts_decoding_and_portions(name, dtype):
+@pytest.mark.parametrize("dtype, page_tokens", [("float32", 4), ("bfloat16", 4), ("bfloat16", 16)])
+def test_whole_prompts_decoding_and_portions(name, dtype, page_tokens):
+    """(Pages of 16 positions: the bfloat16 run's attention on the matrix-core kernels; of 4: on the plain one.)"""
     toks = tokens_for(name, 61, 1)
     want = oracle_logits(model_folder(name), toks)
-    runner = make_runner(name, dtype)
+    runner = make_runner(name, dtype, page_tokens=page_tokens)
     close(run_cut(runner, toks, [61]), want, dtype, "whole")
     close(run_cut(runner, toks, [1]), want, dtype, "token by token")
     close(run_cut(runner, toks, [29, 1]), want, dtype, "prompt, then decoding")
@@ -274,18 +282,20 @@ def test_first_tokens_and_page_sizes(name):
             close(run_cut(runner, toks, [1]), oracle_logits(model_folder(name), toks), "float32", f"{n} tokens, singly")
 
 
-@pytest.mark.parametrize("name, dtype", [("RA", "float32"), ("RC", "float32"), ("RC", "bfloat16"), ("RB", "float32")])
-def test_mixed_batches_with_pages_and_slots_used_again(name, dtype):
+@pytest.mark.parametrize("name, dtype, page_tokens", [("RA", "float32", 4), ("RC", "float32", 4), ("RC", "bfloat16", 4),
+                                                     ("RC", "bfloat16", 8), ("RB", "float32", 4)])
+def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, page_tokens):
     """Five requests of unequal lengths through three slots and a pool that cannot hold them all at once: portions of
     some beside single tokens of others, free pages filled with a huge number."""
     from allpaca_amd.engine.batch import Entry
     rng = np.random.default_rng(9)
     lens = [37, 5, 58, 21, 44]
     reqs = {f"r{i}": tokens_for(name, n, 70 + i) for i, n in enumerate(lens)}
-    runner = make_runner(name, dtype, page_tokens=4, num_pages=34, max_requests=3, poison=True)
+    P_ = page_tokens
+    runner = make_runner(name, dtype, page_tokens=P_, num_pages=34 * 4 // P_, max_requests=3, poison=True)
     waiting, live, at, got = list(reqs), [], {}, {k: [] for k in reqs}
     while waiting or live:
-        while waiting and len(live) < 3 and runner.cache.free_pages(0) >= -(-len(reqs[waiting[0]]) // 4) + 2:
+        while waiting and len(live) < 3 and runner.cache.free_pages(0) >= -(-len(reqs[waiting[0]]) // P_) + 2:
             s = waiting.pop(0)
             runner.admit(s)
             live.append(s)
@@ -311,7 +321,7 @@ def test_mixed_batches_with_pages_and_slots_used_again(name, dtype):
             if at[e.seq] == len(reqs[e.seq]):
                 runner.release(e.seq)
                 live.remove(e.seq)
-    assert runner.cache.paged_groups[0].pool.allocations > 34          # pages came back and went out again
+    assert runner.cache.paged_groups[0].pool.allocations > 34 * 4 // P_          # pages came back and went out again
     for s, toks in reqs.items():
         close(np.concatenate(got[s]), oracle_logits(model_folder(name), toks), dtype, s)
     runner.cache.check()
