@@ -14,7 +14,7 @@
 //                    in attention_bf16.hip, so a row's maximum and sum are registers of 4 lanes.
 //   decoded rows     one row x one kv head x one range of its keys a block: a thread takes a key and forms its score with
 //                    every query head of the group (keys are read once a group), the block's 256 weights a head go
-//                    through LDS, a thread then owns one value element and adds up its keys' values page by page (a
+//                    through LDS, a thread then owns one value element and adds up its keys' values 8 slots at a time (a
 //                    page's slots of an element lie together).  A second kernel adds the ranges and the sink.
 #include "mfma.h"
 #include <math.h>
@@ -262,6 +262,7 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
 // ------------------------------------------------------------------------------------------ decoded rows
 constexpr int DT = 256;       // keys of a pass: one a thread
 constexpr int DMAX = 256;     // largest key and value size
+constexpr int FR = 16;        // 16-byte pieces a thread asks for at a time
 
 // grid: rows x G x n_splits.  Split s of a row takes the keys at positions a0 + s * kps .. a0 + (s + 1) * kps - 1 that
 // the row sees, a0 being the row's first key rounded down to a multiple of DT (kps is a multiple of DT, pages are
@@ -291,7 +292,7 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     const int j = idx / dk, i = idx % dk;
     qs[j * DMAX + i] = bf16_to_float(q[(size_t)r * ldq + (size_t)(g * per + j) * dk + i]) * scale;
   }
-  // the thread's value element and its share of a pass's pages
+  // the thread's value element and its share of a pass's slots
   int dvt = 1;
   while (dvt < dv) dvt <<= 1;
   const int e = tid % dvt, sl = tid / dvt, nsl = DT / dvt;
@@ -302,9 +303,10 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
 
   const int lo_t = a0 + split * kps;
   const int hi_t = min(lo_t + kps, pos + 1);
+  const int nfr = (DT / 8) / nsl;                // 16-byte pieces (8 slots) of this thread's element in a pass
   for (int t0 = lo_t; t0 < hi_t; t0 += DT) {
     if (t0 + DT <= first) continue;             // (only the first pass of the first split can lie in front)
-    // scores of key t0 + tid with every head of the group
+    // scores of key t0 + tid with every head of the group; the key's pieces are asked for together, 16 at a time
     const int t = t0 + tid;
     const bool valid = t >= first && t <= pos;
     float s[HG];
@@ -312,27 +314,51 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     for (int j = 0; j < HG; ++j) s[j] = 0.f;
     if (valid) {
       const bf16_t* kp = head + (size_t)bt[t / P] * page_stride + (size_t)(t % P) * dk;
-      for (int c = 0; c < dk; c += 8) {
-        const Frag kf = load_frag(kp + c);
-        float kv[8];
+      for (int c0 = 0; c0 < dk; c0 += FR * 8) {
+        Frag kf[FR];
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          kv[2 * w] = __uint_as_float(kf.w[w] << 16);
-          kv[2 * w + 1] = __uint_as_float(kf.w[w] & 0xffff0000u);
-        }
+        for (int i = 0; i < FR; ++i)
+          if (c0 + i * 8 < dk) kf[i] = load_frag(kp + c0 + i * 8);
 #pragma unroll
-        for (int j = 0; j < HG; ++j) {
-          if (j < per) {
-            const float4 qa = *reinterpret_cast<const float4*>(qs + j * DMAX + c);
-            const float4 qb = *reinterpret_cast<const float4*>(qs + j * DMAX + c + 4);
-            float a = s[j];
-            a = fmaf(qa.x, kv[0], a); a = fmaf(qa.y, kv[1], a); a = fmaf(qa.z, kv[2], a); a = fmaf(qa.w, kv[3], a);
-            a = fmaf(qb.x, kv[4], a); a = fmaf(qb.y, kv[5], a); a = fmaf(qb.z, kv[6], a); a = fmaf(qb.w, kv[7], a);
-            s[j] = a;
+        for (int i = 0; i < FR; ++i) {
+          if (c0 + i * 8 < dk) {
+            float kv[8];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+              kv[2 * w] = __uint_as_float(kf[i].w[w] << 16);
+              kv[2 * w + 1] = __uint_as_float(kf[i].w[w] & 0xffff0000u);
+            }
+#pragma unroll
+            for (int j = 0; j < HG; ++j) {
+              if (j < per) {
+                const float4 qa = *reinterpret_cast<const float4*>(qs + j * DMAX + c0 + i * 8);
+                const float4 qb = *reinterpret_cast<const float4*>(qs + j * DMAX + c0 + i * 8 + 4);
+                float a = s[j];
+                a = fmaf(qa.x, kv[0], a); a = fmaf(qa.y, kv[1], a); a = fmaf(qa.z, kv[2], a); a = fmaf(qa.w, kv[3], a);
+                a = fmaf(qb.x, kv[4], a); a = fmaf(qb.y, kv[5], a); a = fmaf(qb.z, kv[6], a); a = fmaf(qb.w, kv[7], a);
+                s[j] = a;
+              }
+            }
           }
         }
       }
     }
+    // the first pieces of the thread's value element are asked for now: they do not wait for the weights
+    // piece f of the thread: slots (sl + nsl * f) * 8 .. + 7 of the pass (a piece lies in one page)
+    Frag vf[FR];
+    auto piece_pos = [&](int f) { return t0 + (sl + nsl * f) * 8; };
+    auto load_values = [&](int f0) {
+#pragma unroll
+      for (int i = 0; i < FR; ++i) {
+        const int f = f0 + i;
+        if (f < nfr) {
+          const int tp = piece_pos(f);
+          if (tp <= pos && tp + 8 > first)
+            vf[i] = load_frag(head + (size_t)bt[tp / P] * page_stride + (size_t)P * dk + (size_t)e * P + tp % P);
+        }
+      }
+    };
+    if (e < dv) load_values(0);
 #pragma unroll
     for (int j = 0; j < HG; ++j) {
       if (j < per) {
@@ -368,23 +394,26 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
         o[j] *= alpha[j];
       }
     }
-    // values: element e of the pages sl, sl + nsl, ... of the pass
+    // values: element e at the thread's pieces of the pass
     if (e < dv) {
-      for (int tp = t0 + sl * P; tp < t0 + DT; tp += nsl * P) {
-        if (tp > pos || tp + P <= first) continue;
-        const bf16_t* vp = head + (size_t)bt[tp / P] * page_stride + (size_t)P * dk + (size_t)e * P;
-        for (int c = 0; c < P; c += 8) {
-          const Frag vf = load_frag(vp + c);
+      for (int f0 = 0; f0 < nfr; f0 += FR) {
+        if (f0) load_values(f0);
+#pragma unroll
+        for (int i = 0; i < FR; ++i) {
+          const int f = f0 + i;
+          if (f >= nfr) continue;
+          const int tp = piece_pos(f);
+          if (tp > pos || tp + 8 <= first) continue;
           float vv[8];
 #pragma unroll
           for (int w = 0; w < 4; ++w) {
-            vv[2 * w] = __uint_as_float(vf.w[w] << 16);
-            vv[2 * w + 1] = __uint_as_float(vf.w[w] & 0xffff0000u);
+            vv[2 * w] = __uint_as_float(vf[i].w[w] << 16);
+            vv[2 * w + 1] = __uint_as_float(vf[i].w[w] & 0xffff0000u);
           }
 #pragma unroll
-          for (int i = 0; i < 8; ++i)             // slots the row does not see may hold anything
-            if (tp + c + i < first || tp + c + i > pos) vv[i] = 0.f;
-          const int k0 = tp - t0 + c;
+          for (int k = 0; k < 8; ++k)             // slots the row does not see may hold anything
+            if (tp + k < first || tp + k > pos) vv[k] = 0.f;
+          const int k0 = tp - t0;
 #pragma unroll
           for (int j = 0; j < HG; ++j) {
             if (j < per) {

@@ -1,0 +1,170 @@
+// The short convolution on the heads of projected rows (see plain_mixers.hip for the formulas) for bfloat16 rows, 16
+// bytes a thread: a block takes ROWS consecutive rows whole, a thread PPT pieces of 8 channels of each, with the taps of
+// its channels in registers.  Sums of squares of the pieces go through LDS, so a head may be any multiple of 8 wide.
+// The row holds q heads, then k heads, then v heads.  The state of the convolution is moved on by the plain kernel.
+#include "mfma.h"
+#include <math.h>
+
+namespace {
+
+constexpr int MAXT = 4;   // taps
+constexpr int ROWS = 2;
+
+__device__ __forceinline__ void unpack8(const Frag& f, float* v) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    v[2 * w] = __uint_as_float(f.w[w] << 16);
+    v[2 * w + 1] = __uint_as_float(f.w[w] & 0xffff0000u);
+  }
+}
+
+template <int PPT>
+__global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
+    const bf16_t* __restrict__ proj, int ld, int n_rows, int H, int G, int dk, int dv, const float* __restrict__ bias,
+    const float* __restrict__ conv_w, int taps, const float* __restrict__ state, int width,
+    const int* __restrict__ row_seg, const int* __restrict__ seg_row0, const int* __restrict__ slots,
+    const int* __restrict__ positions, int unit_norm, float eps, bf16_t* __restrict__ q_out, int ldq,
+    const int* __restrict__ block_table, int max_blocks, bf16_t* __restrict__ cache, int P) {
+  extern __shared__ float ssum[];            // [ROWS][pieces]
+  const int tid = threadIdx.x;
+  const int pieces = width / 8;
+  const int r0 = blockIdx.x * ROWS;
+  int seg[ROWS], in_seg[ROWS];
+  const float* st[ROWS];
+#pragma unroll
+  for (int rr = 0; rr < ROWS; ++rr) {
+    const int r = min(r0 + rr, n_rows - 1);
+    seg[rr] = row_seg[r];
+    in_seg[rr] = r - seg_row0[seg[rr]];
+    st[rr] = taps > 1 ? state + (size_t)slots[seg[rr]] * (taps - 1) * width : nullptr;
+  }
+  float y[PPT][ROWS][8];
+#pragma unroll
+  for (int k = 0; k < PPT; ++k) {
+    const int p = tid + 256 * k;
+    if (p >= pieces) continue;
+    const int c0 = p * 8;
+    float b[8], w[8 * MAXT];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] = bias ? bias[c0 + e] : 0.f;
+    if (taps > 1) {
+#pragma unroll
+      for (int j = 0; j < MAXT; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (j < taps) w[j * 8 + e] = conv_w[(size_t)(c0 + e) * taps + j];
+    }
+#pragma unroll
+    for (int rr = 0; rr < ROWS; ++rr) {
+      const int r = min(r0 + rr, n_rows - 1);
+      float acc[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+      for (int j = 0; j < MAXT; ++j) {                 // oldest first, as the plain kernel adds
+        if (j < taps) {
+          const int back = taps - 1 - j;
+          float u[8];
+          if (back <= in_seg[rr]) {
+            unpack8(load_frag(proj + (size_t)(r - back) * ld + c0), u);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) u[e] += b[e];
+          } else {
+            const float* sp = st[rr] + (size_t)(taps - 1 - (back - in_seg[rr])) * width + c0;
+            const float4 a = *reinterpret_cast<const float4*>(sp), c = *reinterpret_cast<const float4*>(sp + 4);
+            u[0] = a.x; u[1] = a.y; u[2] = a.z; u[3] = a.w; u[4] = c.x; u[5] = c.y; u[6] = c.z; u[7] = c.w;
+          }
+          if (taps > 1) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = fmaf(w[j * 8 + e], u[e], acc[e]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = u[e];
+          }
+        }
+      }
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { y[k][rr][e] = acc[e]; ss = fmaf(acc[e], acc[e], ss); }
+      ssum[rr * pieces + p] = ss;
+    }
+  }
+  __syncthreads();
+  const int kq = H * dk, kk = (H + G) * dk;
+#pragma unroll
+  for (int k = 0; k < PPT; ++k) {
+    const int p = tid + 256 * k;
+    if (p >= pieces) continue;
+    const int c0 = p * 8;
+    const int kind = c0 < kq ? 0 : c0 < kk ? 1 : 2;
+    const int d = kind == 2 ? dv : dk;
+    const int rel = c0 - (kind == 0 ? 0 : kind == 1 ? kq : kk);
+    const int head = rel / d, off = rel % d;
+#pragma unroll
+    for (int rr = 0; rr < ROWS; ++rr) {
+      const int r = r0 + rr;
+      if (r >= n_rows) continue;
+      float inv = 1.f;
+      if (unit_norm && kind != 2) {
+        const float* sp = ssum + rr * pieces + (c0 - off) / 8;
+        float ss = 0.f;
+        for (int i = 0; i < d / 8; ++i) ss += sp[i];
+        inv = 1.0f / sqrtf(ss / (float)d + eps);
+      }
+      Frag o;
+#pragma unroll
+      for (int wd = 0; wd < 4; ++wd) o.w[wd] = pack_bf16x2(y[k][rr][2 * wd] * inv, y[k][rr][2 * wd + 1] * inv);
+      if (kind == 0) {
+        *reinterpret_cast<Frag*>(q_out + (size_t)r * ldq + c0) = o;
+        continue;
+      }
+      const int pos = positions[r];
+      const int page = block_table[(size_t)seg[rr] * max_blocks + pos / P];
+      bf16_t* base = cache + ((size_t)page * G + head) * (size_t)P * (dk + dv);
+      if (kind == 1) {
+        *reinterpret_cast<Frag*>(base + (size_t)(pos % P) * dk + off) = o;
+      } else {
+        bf16_t* vp = base + (size_t)P * dk + (size_t)off * P + (pos % P);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vp[(size_t)e * P] = (bf16_t)((e & 1) ? (o.w[e / 2] >> 16) : (o.w[e / 2] & 0xffffu));
+      }
+    }
+  }
+}
+
+}  // namespace
+
+// 1 if the kernel takes these sizes (q, k and v heads side by side from column 0 on), else 0
+APC_EXPORT int apc_conv_heads_bf16_takes(int ld, int width, int H, int G, int dk, int dv, int taps, int ldq) {
+  if (H <= 0 || G < 0 || dk % 8 || (G && dv % 8) || taps < 1 || taps > MAXT || ld % 8 || ldq % 8) return 0;
+  if (width != H * dk + G * (dk + dv) || width / 8 > 8 * 256) return 0;
+  return 1;
+}
+
+APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, int G, int dk, int dv, const float* bias,
+                                   const float* conv_w, int taps, const float* state, int width, const int* row_seg,
+                                   const int* seg_row0, const int* slots, const int* positions, int unit_norm, float eps,
+                                   void* q_out, int ldq, const int* block_table, int max_blocks, void* cache,
+                                   int page_tokens, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (!apc_conv_heads_bf16_takes(ld, width, H, G, dk, dv, taps, ldq)) return APC_ERR_UNSUPPORTED;
+  if (((uintptr_t)proj & 15u) || ((uintptr_t)q_out & 15u) || ((uintptr_t)cache & 15u) || ((uintptr_t)state & 15u))
+    return APC_ERR_UNSUPPORTED;
+  if (taps > 1 && (!conv_w || !state || !slots)) return APC_ERR_BAD_ARG;
+  if (G > 0 && (!cache || !block_table || page_tokens <= 0 || max_blocks <= 0)) return APC_ERR_BAD_ARG;
+  const int pieces = width / 8;
+  const int ppt = (pieces + 255) / 256;
+  dim3 grid((n_rows + ROWS - 1) / ROWS), block(256);
+  const size_t lds = (size_t)ROWS * pieces * sizeof(float);
+#define CH_LAUNCH(PPT_)                                                                                               \
+  hipLaunchKernelGGL((conv_heads_bf16_kernel<PPT_>), grid, block, lds, stream, (const bf16_t*)proj, ld, n_rows, H, G, \
+                     dk, dv, bias, conv_w, taps, state, width, row_seg, seg_row0, slots, positions, unit_norm, eps,    \
+                     (bf16_t*)q_out, ldq, block_table, max_blocks, (bf16_t*)cache, page_tokens)
+  if (ppt <= 1) CH_LAUNCH(1);
+  else if (ppt <= 2) CH_LAUNCH(2);
+  else if (ppt <= 4) CH_LAUNCH(4);
+  else CH_LAUNCH(8);
+#undef CH_LAUNCH
+  APC_LAUNCH_CHECK();
+  return 0;
+}

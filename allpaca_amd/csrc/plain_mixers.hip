@@ -137,6 +137,18 @@ APC_EXPORT int apc_conv_heads(const void* proj, int in_dtype, int ld, int q_off,
   return 0;
 }
 
+// The second half alone: for callers that ran the first half on another kernel.
+APC_EXPORT int apc_conv_state(const void* proj, int in_dtype, int ld, const float* bias, int taps, float* state,
+                              int width, int n_segs, const int* seg_row0, const int* seg_rows, const int* slots,
+                              hipStream_t stream) {
+  if (n_segs <= 0 || taps <= 1) return 0;
+  if (!state || width <= 0 || taps > MAX_TAPS || n_segs > 65535) return APC_ERR_BAD_ARG;
+  hipLaunchKernelGGL(conv_state_kernel, dim3(ceil_div(width, 256), n_segs), dim3(256), 0, stream, proj, in_dtype, ld,
+                     bias, taps, state, width, seg_row0, seg_rows, slots);
+  APC_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------------------
 // Attention over pages with a mask and an optional sink: one wave per (query row, head), keys in order in groups of
 // 64 anchored at key 0, online softmax in float32.
@@ -299,6 +311,106 @@ __global__ __launch_bounds__(NT) void streams_step_kernel(float* __restrict__ x,
   }
 }
 
+// The same for widths that are a multiple of 4 and at most NT * 4 * VPT, 16 bytes a load: what a thread reads of the
+// row stays in registers between the sum of squares and the scaling.  Which of the two kernels runs is fixed by the
+// width and the alignment alone, never by the batch.
+template <int NT, int VPT>
+__global__ __launch_bounds__(NT) void streams_step_f4_kernel(float* __restrict__ x, int S, int D,
+                                                             const void* __restrict__ y, int y_dtype, int ldy,
+                                                             const float* __restrict__ mix,
+                                                             const float* __restrict__ out_w,
+                                                             const float* __restrict__ in_w,
+                                                             const float* __restrict__ norm_w, float eps,
+                                                             void* __restrict__ h, int h_dtype, int ldh,
+                                                             const int* __restrict__ rows) {
+  __shared__ float red[NT / WAVE];
+  __shared__ float w_mix[MAX_STREAMS * MAX_STREAMS], w_out[MAX_STREAMS], w_in[MAX_STREAMS];
+  const int r = blockIdx.x;
+  const size_t t = rows ? (size_t)rows[r] : (size_t)r;
+  float* xr = x + t * (size_t)S * D;
+  if (threadIdx.x < S * S && y) w_mix[threadIdx.x] = mix[threadIdx.x];
+  if (threadIdx.x < S) {
+    if (y) w_out[threadIdx.x] = out_w[threadIdx.x];
+    if (in_w) w_in[threadIdx.x] = in_w[threadIdx.x];
+  }
+  __syncthreads();
+  const int n4 = D / 4;
+  float4 u[VPT];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int i = threadIdx.x + k * NT;
+    u[k] = float4{0.f, 0.f, 0.f, 0.f};
+    if (i >= n4) continue;
+    float4 v[MAX_STREAMS];
+#pragma unroll
+    for (int a = 0; a < MAX_STREAMS; ++a)
+      if (a < S) v[a] = reinterpret_cast<const float4*>(xr + (size_t)a * D)[i];
+    if (y) {
+      float4 yy;
+      if (y_dtype == APC_F32) {
+        yy = reinterpret_cast<const float4*>((const float*)y + t * ldy)[i];
+      } else {
+        const uint2 p = reinterpret_cast<const uint2*>((const bf16_t*)y + t * ldy)[i];
+        yy = float4{__uint_as_float(p.x << 16), __uint_as_float(p.x & 0xffff0000u), __uint_as_float(p.y << 16),
+                    __uint_as_float(p.y & 0xffff0000u)};
+      }
+      float4 nv[MAX_STREAMS];
+#pragma unroll
+      for (int b = 0; b < MAX_STREAMS; ++b) {
+        if (b < S) {
+          float4 acc = float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int a = 0; a < MAX_STREAMS; ++a) {
+            if (a < S) {
+              const float m = w_mix[a * S + b];
+              acc.x = fmaf(m, v[a].x, acc.x); acc.y = fmaf(m, v[a].y, acc.y);
+              acc.z = fmaf(m, v[a].z, acc.z); acc.w = fmaf(m, v[a].w, acc.w);
+            }
+          }
+          const float o = w_out[b];
+          nv[b] = float4{fmaf(o, yy.x, acc.x), fmaf(o, yy.y, acc.y), fmaf(o, yy.z, acc.z), fmaf(o, yy.w, acc.w)};
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < MAX_STREAMS; ++b)
+        if (b < S) { v[b] = nv[b]; reinterpret_cast<float4*>(xr + (size_t)b * D)[i] = nv[b]; }
+    }
+    if (in_w) {
+      float4 acc = float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int a = 0; a < MAX_STREAMS; ++a) {
+        if (a < S) {
+          const float m = w_in[a];
+          acc.x = fmaf(m, v[a].x, acc.x); acc.y = fmaf(m, v[a].y, acc.y);
+          acc.z = fmaf(m, v[a].z, acc.z); acc.w = fmaf(m, v[a].w, acc.w);
+        }
+      }
+      u[k] = acc;
+      ss = fmaf(acc.x, acc.x, ss); ss = fmaf(acc.y, acc.y, ss); ss = fmaf(acc.z, acc.z, ss); ss = fmaf(acc.w, acc.w, ss);
+    }
+  }
+  if (!in_w) return;
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int i = threadIdx.x + k * NT;
+    if (i >= n4) continue;
+    float4 g = float4{1.f, 1.f, 1.f, 1.f};
+    if (norm_w) g = reinterpret_cast<const float4*>(norm_w)[i];
+    const float4 o = float4{(u[k].x * inv) * g.x, (u[k].y * inv) * g.y, (u[k].z * inv) * g.z, (u[k].w * inv) * g.w};
+    if (h_dtype == APC_F32) {
+      reinterpret_cast<float4*>((float*)h + (size_t)r * ldh)[i] = o;
+    } else {
+      uint2 p;
+      p.x = pack_bf16x2(o.x, o.y);
+      p.y = pack_bf16x2(o.z, o.w);
+      reinterpret_cast<uint2*>((bf16_t*)h + (size_t)r * ldh)[i] = p;
+    }
+  }
+}
+
 APC_EXPORT int apc_streams_step(float* x, int n_rows, int S, int D, const void* y, int y_dtype, int ldy,
                                 const float* mix, const float* out_w, const float* in_w, const float* norm_w, float eps,
                                 void* h, int h_dtype, int ldh, const int* rows, hipStream_t stream) {
@@ -307,6 +419,20 @@ APC_EXPORT int apc_streams_step(float* x, int n_rows, int S, int D, const void* 
       (rows && y))
     return APC_ERR_BAD_ARG;
   if (S > MAX_STREAMS) return APC_ERR_UNSUPPORTED;
+  const bool wide = D % 4 == 0 && D <= 256 * 4 * 8 && !((uintptr_t)x & 15u) && !((uintptr_t)norm_w & 15u) &&
+                    (!y || (ldy % 4 == 0 && !((uintptr_t)y & 15u))) && (!in_w || (ldh % 4 == 0 && !((uintptr_t)h & 15u)));
+  if (wide) {
+#define ST_LAUNCH(VPT_)                                                                                              \
+  hipLaunchKernelGGL((streams_step_f4_kernel<256, VPT_>), dim3(n_rows), dim3(256), 0, stream, x, S, D, y, y_dtype, ldy, \
+                     mix, out_w, in_w, norm_w, eps, h, h_dtype, ldh, rows)
+    if (D <= 1024) ST_LAUNCH(1);
+    else if (D <= 2048) ST_LAUNCH(2);
+    else if (D <= 4096) ST_LAUNCH(4);
+    else ST_LAUNCH(8);
+#undef ST_LAUNCH
+    APC_LAUNCH_CHECK();
+    return 0;
+  }
   hipLaunchKernelGGL(streams_step_kernel<256>, dim3(n_rows), dim3(256), 0, stream, x, S, D, y, y_dtype, ldy, mix, out_w,
                      in_w, norm_w, eps, h, h_dtype, ldh, rows);
   APC_LAUNCH_CHECK();

@@ -35,6 +35,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_gemm_plain": [P, I, I, P, I, I, P, I, I, I, I, I, I, P],
         "apc_paged_attention_plain": [P, I, I, I, P, I, I, I, I, I, I, P, I, I, P, I, P, P, I, F, P],
         "apc_conv_heads": [P, I, I, I, I, I, I, I, I, I, I, I, P, P, I, P, I, P, P, P, P, P, I, F, P, I, I, P, I, P, I, I, P],
+        "apc_conv_state": [P, I, I, P, I, P, I, I, P, P, P, P],
         "apc_masked_attention_plain": [P, I, I, P, I, I, I, I, I, I, I, P, I, I, P, I, P, P, I, I, I, F, P],
         "apc_streams_step": [P, I, I, I, P, I, I, P, P, P, P, F, P, I, I, P, P],
         "apc_embed_streams": [P, I, P, P, F, P, I, I, I, P],
@@ -65,6 +66,8 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_skinny_swiglu_bf16": [P, I, P, P, P, I, I, I, I, P],
         "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, F, I, I, P, P],
         "apc_attention_decode_bf16": [P, I, I, P, I, I, I, I, I, P, I, P, I, P, P, P, I, F, I, I, P, P, P],
+        "apc_conv_heads_bf16_takes": [I, I, I, I, I, I, I, I],
+        "apc_conv_heads_bf16": [P, I, I, I, I, I, I, P, P, I, P, I, P, P, P, P, I, F, P, I, P, I, P, I, P],
         "apc_attention_masked_takes": [I, I, I, I, I],
         "apc_attention_masked_prefill_bf16": [P, I, P, I, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, F, P],
         "apc_attention_masked_decode_bf16": [P, I, P, I, I, I, I, I, I, P, I, P, I, P, P, P, I, I, I, F, I, I, P, P],
@@ -114,7 +117,7 @@ class KernelTimer:
 
 _timer = None
 # entry points that launch nothing (questions about sizes): never timed
-NOT_KERNELS = {"apc_attention_masked_takes", "apc_attention_decode_whole_fits", "apc_attention_decode_last_fits", "apc_attention_prefill_tile_rows",
+NOT_KERNELS = {"apc_attention_masked_takes", "apc_conv_heads_bf16_takes", "apc_attention_decode_whole_fits", "apc_attention_decode_last_fits", "apc_attention_prefill_tile_rows",
                "apc_attention_prefill_wide_takes",
                "apc_gemm_direct_k_split", "apc_gemm_direct_emit_parts", "apc_sample_rows_scratch_kib"}
 

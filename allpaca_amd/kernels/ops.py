@@ -408,6 +408,28 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
         max_blocks = block_table.shape[1]
     S = step.n_segs
     L = _lib.load("plain")
+    if (_tuned_ok(proj, q_out) and (cache is None or cache.dtype == torch.bfloat16) and q_off == 0
+            and (G == 0 or (k_off == n_heads * key_dim and v_off == (n_heads + G) * key_dim))):
+        LT = _lib.load("tuned")
+        if (LT.apc_conv_heads_bf16_takes(ld, width, n_heads, G, key_dim, value_dim, taps, ldq)
+                and proj.data_ptr() % 16 == 0 and q_out.data_ptr() % 16 == 0
+                and (cache is None or cache.data_ptr() % 16 == 0) and (state is None or state.data_ptr() % 16 == 0)
+                and (taps == 1 or width % 4 == 0)):
+            # the same on 16 bytes a thread (library `tuned`); the plain kernel then moves the state on
+            _lib.check(LT.apc_conv_heads_bf16(
+                proj.data_ptr(), ld, T, n_heads, G, key_dim, value_dim, _f32(bias, width, "bias"),
+                _f32(conv_w, width * taps, "conv weights") if taps > 1 else 0, taps,
+                state.data_ptr() if taps > 1 else 0, width, _i32(step.row_seg, T, "row_seg"),
+                _i32(step.seg_row0, S, "seg_row0"), _i32(slots, S, "slots") if taps > 1 else 0,
+                _i32(step.positions, T, "positions"), 1 if unit_norm else 0, float(eps), q_out.data_ptr(), ldq,
+                block_table.data_ptr() if G else 0, max_blocks, cache.data_ptr() if G else 0, page_tokens, _stream()),
+                "conv_heads_bf16")
+            if taps > 1:
+                _lib.check(L.apc_conv_state(proj.data_ptr(), _code(proj), ld, _f32(bias, width, "bias"), taps,
+                                            state.data_ptr(), width, S, _i32(step.seg_row0, S, "seg_row0"),
+                                            _i32(step.seg_rows, S, "seg_rows"), _i32(slots, S, "slots"), _stream()),
+                           "conv_state")
+            return
     _lib.check(L.apc_conv_heads(
         proj.data_ptr(), _code(proj), ld, q_off, k_off, v_off, T, S, n_heads, G, key_dim, value_dim,
         _f32(bias, width, "bias"), _f32(conv_w, width * taps, "conv weights") if taps > 1 else 0, taps,
@@ -509,18 +531,12 @@ def clamped_glu_mul(gate_up: torch.Tensor, out: torch.Tensor, alpha: float, limi
 
 def clamped_glu(h: torch.Tensor, w_gate_up, out: torch.Tensor, alpha: float, limit: float) -> None:
     """out[t, f] = g * sigmoid(alpha g) * (u + 1), g = min(h . Wg[f], limit), u = clamp(h . Wu[f], -limit, limit);
-    w_gate_up is [Wg; Wu] of shape [2F, D], or the pair of their tiled forms."""
+    w_gate_up is [Wg; Wu] of shape [2F, D] (row-major or tiled): one product for both branches (in the run's element
+    type: 16 bits in a bfloat16 run), then the activation."""
     T, F = out.shape
-    if isinstance(w_gate_up, tuple):
-        from . import tuned
-        if tuned.clamped_glu_bf16(h, w_gate_up[0], w_gate_up[1], out, alpha, limit):
-            return
-        gu = torch.empty((T, 2 * F), dtype=torch.float32, device=h.device)
-        tuned.gemm_bf16(h, w_gate_up[0], gu[:, :F])
-        tuned.gemm_bf16(h, w_gate_up[1], gu[:, F:])
-    else:
-        gu = torch.empty((T, 2 * F), dtype=torch.float32, device=h.device)
-        gemm_plain(h, w_gate_up, gu)
+    packed = isinstance(w_gate_up, PackedWeight)
+    gu = torch.empty((T, 2 * F), dtype=h.dtype if packed else torch.float32, device=h.device)
+    linear(h, w_gate_up, gu)
     clamped_glu_mul(gu, out, alpha, limit)
 
 

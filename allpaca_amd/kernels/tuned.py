@@ -499,8 +499,3 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
             int(mask_size), 1 if sink else 0, float(scale), splits, kps, parts.data_ptr(), stream),
             "attention_masked_decode_bf16")
     return True
-
-
-def clamped_glu_bf16(h, wg: PackedWeight, wu: PackedWeight, out, alpha: float, limit: float) -> bool:
-    """The clamped gated activation in the epilogue of the gate and up products; False where there is no kernel."""
-    return False

@@ -81,8 +81,8 @@ class ClampedGLU(FeedForward):
         n = self.names
         g, u = tensors[n["gate"]], tensors[n["up"]]
         dt = g.dtype if g.dtype == u.dtype else torch.float32
-        wg, wu = ops.prepare_matrix(to_device(g, rt, dt), rt.dtype), ops.prepare_matrix(to_device(u, rt, dt), rt.dtype)
-        self.w_gate_up = torch.cat([wg, wu], dim=0).contiguous() if isinstance(wg, torch.Tensor) else (wg, wu)
+        # one [2F, D] matrix (gate rows, then up rows): a single product gives both branches of a row
+        self.w_gate_up = ops.prepare_matrix(torch.cat([to_device(g, rt, dt), to_device(u, rt, dt)], dim=0), rt.dtype)
         self.w_down = ops.prepare_matrix(to_device(tensors[n["down"]], rt), rt.dtype)
 
     def forward(self, h, step) -> torch.Tensor:

@@ -28,7 +28,7 @@ PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
 def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, use_graphs=True, max_context=0,
-                 chunk_tokens=2048, pool_tokens=0):
+                 chunk_tokens=2048, pool_tokens=0, set_layers=True):
     """An engine on random weights made directly on the GPU (no model folder is written for 16 GB)."""
     import torch
 
@@ -38,7 +38,8 @@ def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, 
     from allpaca_amd.parts import Runtime
     from allpaca_amd.weights import random_tensors
 
-    cfg_json = dict(cfg_json, num_hidden_layers=layers)
+    if set_layers:
+        cfg_json = dict(cfg_json, num_hidden_layers=layers)
     _, cfg, spec = describe_model(cfg_json)
     model = DecoderModel(spec)
     tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
@@ -431,6 +432,163 @@ def sampler_times(vocab: int) -> dict:
     return out
 
 
+# ---- the Risizen design beside the llama decoder at equal sizes ---------------------------------------------------
+# name -> width, heads, kv heads, head size (keys and values alike), feed-forward width, vocabulary
+DESIGN_SIZES = {"1b": (2048, 32, 8, 64, 8192, 128256), "8b": (4096, 32, 8, 128, 14336, 128256)}
+# entry points of the new design -> the like entry points of the llama decoder
+LIKE_KERNELS = {
+    "apc_conv_heads": ["apc_rope_kv_write_bf16", "apc_rope_kv_write"],
+    "apc_attention_masked_prefill_bf16": ["apc_attention_prefill_bf16"],
+    "apc_attention_masked_decode_bf16": ["apc_attention_decode_bf16"],
+    "apc_streams_step": ["apc_rmsnorm_rows"],
+    "apc_embed_streams": ["apc_embed_rows", "apc_embed_rows_tiled"],
+    "apc_clamped_glu": ["apc_gemm_swiglu_bf16", "apc_skinny_swiglu_bf16", "apc_skinny_swiglu_pre_bf16"],
+}
+
+
+def design_configs(size: str, layers: int, chunk: int, streams: int = 2, taps: int = 4):
+    D, H, G, d, F, V = DESIGN_SIZES[size]
+    mixer = dict(heads=H, kv_heads=G, dim=d, vdim=d, scale=d ** -0.5, conv=taps, mask=dict(size=chunk))
+    risizen = dict(architecture="Risizen", vocab=V, width=D, streams=streams, norm=dict(eps=1e-6), logit_scale=1.0,
+                   layers=[dict(type="attention", mixer=dict(mixer), mlp=dict(kind="dense", ff=F, limit=7.0))
+                           for _ in range(layers)])
+    llama = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=V, hidden_size=D,
+                 num_hidden_layers=layers, num_attention_heads=H, num_key_value_heads=G, head_dim=d,
+                 intermediate_size=F, rms_norm_eps=1e-6, rope_theta=500000.0, rope_scaling=None,
+                 tie_word_embeddings=False, max_position_embeddings=8192, hidden_act="silu")
+    return {"risizen": risizen, "llama": llama}
+
+
+def design_point(cfg_json, dtype, batch, context, steps, warmup, T):
+    """Prefill tok/s (one prompt of T tokens in one step), decode tok/s (batch x context, graphs) and the time of
+    every kernel in an eager prefill step and an eager decode step of one model."""
+    import numpy as np
+    import torch
+
+    from allpaca_amd.engine.batch import Entry
+    from allpaca_amd.kernels import lib as klib
+    from allpaca_amd.sampling import GenerationParams
+    extra = warmup + steps + decode_during_prefill(batch, context) + 16
+    _, eng = build_engine(cfg_json, dtype, batch + 1, context, extra, 0, max_context=context + extra, set_layers=False)
+    V = eng.model.spec.vocab_size
+    rng = np.random.default_rng(0)
+    r = eng.runner
+
+    def prefill_once(tag):
+        toks = rng.integers(0, V, size=T).tolist()
+        r.admit(tag)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        r.step([Entry(tag, toks, [T - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        r.release(tag)
+        return dt
+
+    prefill_once("w")
+    psec = min(prefill_once(("p", i)) for i in range(3))
+    native, r.native = r.native, None          # the timers sit around the entry points as Python calls them
+    with klib.timing() as t:
+        prefill_once("k")
+    prefill_kernels = {k: round(v["us"], 1) for k, v in t.totals().items()}
+    r.native = native
+    gp = GenerationParams(max_tokens=extra, temperature=0.0)
+    for _ in range(batch):
+        eng.add_request(rng.integers(0, V, size=context - 1).tolist(), gp)
+    while any(not q.decoding for q in eng.scheduler.running) or eng.scheduler.waiting:
+        eng.step()
+    for _ in range(warmup):
+        eng.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        eng.step()
+    torch.cuda.synchronize()
+    dsec = (time.perf_counter() - t0) / steps
+    # one eager decode step of as many rows at the same context, under the timers (requests of their own)
+    for q in list(eng.scheduler.running):
+        eng.abort(q.id)
+    eng.step()
+    torch.cuda.synchronize()
+    ids = [("d", i) for i in range(batch)]
+    native, r.native = r.native, None
+    graphs, r.use_graphs = r.use_graphs, False
+    for i in ids:
+        r.admit(i)
+        r.step([Entry(i, rng.integers(0, V, size=context).tolist(), [])])
+    entries = [Entry(i, [1], [0]) for i in ids]
+    r.step(entries)
+    with klib.timing() as t:
+        r.step(entries)
+    decode_kernels = {k: round(v["us"], 1) for k, v in t.totals().items()}
+    r.native, r.use_graphs = native, graphs
+    out = {"prefill_tok_s": round(T / psec, 1), "prefill_ms": round(psec * 1e3, 3),
+           "decode_tok_s": round(batch / dsec, 1), "decode_ms_per_step": round(dsec * 1e3, 4),
+           "weight_bytes": weight_bytes(eng), "prefill_kernels_us": prefill_kernels, "decode_kernels_us": decode_kernels}
+    del eng, r
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
+
+
+def design_rooflines(size, layers, streams, batch, context, T, points):
+    """For the kernels the new design adds and their like kernels of the llama decoder: the bytes or the arithmetic
+    of the launches of a step, over the measured time, as a share of the card's peak (8 TB/s, 2.5 PFLOP/s)."""
+    D, H, G, d, F, V = DESIGN_SIZES[size]
+    qkv = (H + 2 * G) * d
+
+    def work(name, rows, keys_sum):
+        """(bytes, flops) of all of a step's launches of entry point `name`."""
+        if name in ("apc_conv_heads", "apc_rope_kv_write_bf16", "apc_rope_kv_write"):
+            return layers * rows * (qkv + H * d + 2 * G * d) * 2, 0       # rows read, q and the pages' rows written
+        if name in ("apc_attention_masked_prefill_bf16", "apc_attention_prefill_bf16"):
+            return 0, layers * 4 * keys_sum * H * d
+        if name in ("apc_attention_masked_decode_bf16", "apc_attention_decode_bf16"):
+            return layers * keys_sum * G * 2 * d * 2, 0
+        if name == "apc_streams_step":       # per sublayer: the streams read and written, the output read, h written
+            return layers * 2 * rows * (2 * streams * D * 4 + D * 4 + D * 2), 0
+        return None
+
+    table = {}
+    for phase, rows, keys_sum in (("prefill", T, T * (T + 1) // 2), ("decode", batch, batch * context)):
+        for new, likes in LIKE_KERNELS.items():
+            row = {}
+            for model, names in (("risizen", [new]), ("llama", likes)):
+                us = sum(points[model][phase + "_kernels_us"].get(n, 0.0) for n in names)
+                name = next((n for n in names if n in points[model][phase + "_kernels_us"]), None)
+                if not us or name is None:
+                    continue
+                w = work(name, rows, keys_sum)
+                row[model] = {"us": round(us, 1)}
+                if w:
+                    row[model]["share_of_peak"] = round(max(w[0] / (us * 1e-6) / (HBM_PEAK_GBS * 1e9),
+                                                            w[1] / (us * 1e-6) / PEAK_FLOPS["bf16"]), 4)
+            if row:
+                table[f"{phase}: {new}"] = row
+    return table
+
+
+def design_run(args) -> int:
+    layers = args.layers or 4
+    T, batch, context = 2048, args.batch, args.context
+    out = {"metric": "Risizen beside the llama decoder at equal sizes: prefill tok/s (one prompt of 2048 tokens) and "
+                     f"decode tok/s (batch {batch}, context {context})", "unit": "tok/s", "n_gpus": 1,
+           "dtype": args.dtype, "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
+           "config": {"layers": layers, "streams": 2, "conv_taps": 4, "chunk": 2 * context, "page_tokens": 16},
+           "sizes": {}}
+    for size in args.design_sizes.split(","):
+        cfgs = design_configs(size, layers, 2 * context)
+        points = {m: design_point(c, args.dtype, batch, context, args.steps, args.warmup, T) for m, c in cfgs.items()}
+        out["sizes"][size] = {
+            "shape": dict(zip(("width", "heads", "kv_heads", "head_size", "ff", "vocab"), DESIGN_SIZES[size])),
+            **points,
+            "prefill_risizen_over_llama": round(points["risizen"]["prefill_tok_s"] / points["llama"]["prefill_tok_s"], 3),
+            "decode_risizen_over_llama": round(points["risizen"]["decode_tok_s"] / points["llama"]["decode_tok_s"], 3),
+            "like_kernels": design_rooflines(size, layers, 2, batch, context, T, points)}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -466,6 +624,10 @@ def main() -> int:
                     help="for profiling: only the decode steps at --batch (as --no-points), only the 2,048-token "
                          "prefill (prints its figures as the line's value), or only the sampler over the preset's "
                          "vocabulary (microseconds a step's rows take on the GPU and on the host)")
+    ap.add_argument("--design", choices=["risizen"], default=None,
+                    help="instead of the default workload: the named design beside the llama decoder at equal sizes "
+                         "(--design-sizes), prefill and decode throughput and the times of their like kernels")
+    ap.add_argument("--design-sizes", default="1b,8b", help="with --design: sizes of the comparison, of " + ",".join(DESIGN_SIZES))
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
@@ -481,6 +643,8 @@ def main() -> int:
     klib.load("plain")
     klib.load("tuned")
 
+    if args.design:
+        return design_run(args)
     if args.kernel_times:
         print(json.dumps({"metric": "microseconds per kernel and step (event timers, eager passes)", "unit": "us",
                           "n_gpus": 1, "dtype": args.dtype,

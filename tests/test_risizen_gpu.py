@@ -174,7 +174,7 @@ def test_one_key_stands_out(mask, size, pos, key, seen, rows, dtype):
     assert hit == seen, (last[0, :3], seen)
 
 
-@pytest.mark.parametrize("S, D", [(1, 40), (2, 192), (3, 1000), (4, 64)])
+@pytest.mark.parametrize("S, D", [(1, 40), (2, 192), (3, 1000), (4, 64), (2, 50), (3, 4100), (8, 8192)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_streams_read_write_and_both(S, D, dtype):
     from allpaca_amd.kernels import ops
