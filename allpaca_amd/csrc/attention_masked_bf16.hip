@@ -12,10 +12,9 @@
 //                    v_mfma_f32_16x16x32_bf16; keys and values in tiles of 64 through LDS; online softmax whose running
 //                    maximum starts at the sink's score.  The products are transposed (S^T = K Q^T, O^T = V^T P^T), as
 //                    in attention_bf16.hip, so a row's maximum and sum are registers of 4 lanes.
-//   decoded rows     one row x one kv head x one range of its keys a block: a thread takes a key and forms its score with
-//                    every query head of the group (keys are read once a group), the block's 256 weights a head go
-//                    through LDS, a thread then owns one value element and adds up its keys' values 8 slots at a time (a
-//                    page's slots of an element lie together).  A second kernel adds the ranges and the sink.
+//   decoded rows     one row x one kv head x one range of its keys a block; the query heads of the group are the 16
+//                    columns of an MFMA tile, so keys and values are read once a group, straight from the pages into
+//                    the operands.  A second kernel adds the ranges and the sink.
 #include "mfma.h"
 #include <math.h>
 
@@ -260,27 +259,36 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
 }
 
 // ------------------------------------------------------------------------------------------ decoded rows
-constexpr int DT = 256;       // keys of a pass: one a thread
+constexpr int DT = 256;       // keys of a pass: one a thread in the softmax
 constexpr int DMAX = 256;     // largest key and value size
-constexpr int FR = 16;        // 16-byte pieces a thread asks for at a time
+constexpr int HGMAX = 16;     // query heads of a kv head: the 16 columns of an MFMA tile
+constexpr int SROW = DT + 4;  // floats of a row of scores in LDS (heads then fall into different banks)
+constexpr int PROW = DT + 8;  // bfloat16 of a row of weights in LDS
 
 // grid: rows x G x n_splits.  Split s of a row takes the keys at positions a0 + s * kps .. a0 + (s + 1) * kps - 1 that
 // the row sees, a0 being the row's first key rounded down to a multiple of DT (kps is a multiple of DT, pages are
-// powers of two up to DT: a pass starts at a page's first slot).  It leaves, per query head of the group, the maximum
-// score m, sum exp(s - m) and sum exp(s - m) v of its keys in `parts` [row][head][split][2 + dv].
-template <int HG>  // query heads of a kv head, rounded up to a power of two
+// powers of two up to DT: 8 consecutive positions from a multiple of 8 on lie in one page).  It leaves, per query head
+// of the group, the maximum score m, sum exp(s - m) and sum exp(s - m) v of its keys in `parts`
+// [row][head][split][2 + dv].
+// A pass of 256 keys: wave w forms the scores of keys 64 w .. 64 w + 63 with all heads of the group (S = K Q^T, keys
+// as the rows of the tile, straight from the pages), the block takes maxima and sums with a key a thread, the weights go
+// to LDS in bfloat16, and wave w adds up value elements 16 (w + 4 i) .. + 15 over all 256 keys (O^T = V^T P^T, 8 slots of
+// an element a lane, straight from the pages).
+template <int KS, int ET>  // 32-element steps over a key; value tiles of 16 elements a wave
 __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     const bf16_t* __restrict__ q, int ldq, int H, int G, int dk, int dv, const bf16_t* __restrict__ cache, int P,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ positions,
     const int* __restrict__ row_seg, const int* __restrict__ rows, int mask, int mask_size, float scale, int n_splits,
     int kps, float* __restrict__ parts) {
-  __shared__ __attribute__((aligned(16))) float qs[HG * DMAX];
-  __shared__ __attribute__((aligned(16))) float ps[HG * DT];
-  __shared__ float red[2][HG][DT / WAVE];
+  __shared__ __attribute__((aligned(16))) float sc[HGMAX * SROW];
+  __shared__ __attribute__((aligned(16))) bf16_t ps[HGMAX * PROW];
+  __shared__ float red[2][HGMAX][DT / WAVE];
+  __shared__ float al[HGMAX];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  const int li = lane % 16, lc = lane / 16;
   const int split = blockIdx.x % n_splits, g = (blockIdx.x / n_splits) % G, ri = blockIdx.x / (n_splits * G);
   const int r = rows ? rows[ri] : ri;
-  const int per = H / G;                        // query heads of this kv head (<= HG)
+  const int per = H / G;                        // query heads of this kv head (<= HGMAX)
   const int pos = positions[r];
   const int first = first_seen(pos, mask, mask_size);
   const int a0 = (first / DT) * DT;
@@ -288,161 +296,130 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
   const size_t page_stride = (size_t)G * P * (dk + dv);
   const bf16_t* head = cache + (size_t)g * P * (dk + dv);
 
-  for (int idx = tid; idx < per * dk; idx += DT) {
-    const int j = idx / dk, i = idx % dk;
-    qs[j * DMAX + i] = bf16_to_float(q[(size_t)r * ldq + (size_t)(g * per + j) * dk + i]) * scale;
-  }
-  // the thread's value element and its share of a pass's slots
-  int dvt = 1;
-  while (dvt < dv) dvt <<= 1;
-  const int e = tid % dvt, sl = tid / dvt, nsl = DT / dvt;
-  float m_run[HG], l_run[HG], o[HG];
+  // the heads' queries as the second operand: column li = head, 8 elements from (ks * 32 + lc * 8) on
+  Frag qf[KS];
 #pragma unroll
-  for (int j = 0; j < HG; ++j) { m_run[j] = -INFINITY; l_run[j] = 0.f; o[j] = 0.f; }
-  __syncthreads();
+  for (int ks = 0; ks < KS; ++ks) {
+    const int c = ks * 32 + lc * 8;
+    qf[ks] = (li < per && c < dk) ? load_frag(q + (size_t)r * ldq + (size_t)(g * per + li) * dk + c) : zero_frag();
+  }
+  for (int idx = tid; idx < HGMAX * PROW; idx += DT) ps[idx] = 0;    // rows of heads that do not exist stay 0
+  float m_run[HGMAX], l_run[HGMAX];
+#pragma unroll
+  for (int j = 0; j < HGMAX; ++j) { m_run[j] = -INFINITY; l_run[j] = 0.f; }
+  floatx4 o[ET];
+#pragma unroll
+  for (int i = 0; i < ET; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int n_et = (dv + 15) / 16;
 
   const int lo_t = a0 + split * kps;
   const int hi_t = min(lo_t + kps, pos + 1);
-  const int nfr = (DT / 8) / nsl;                // 16-byte pieces (8 slots) of this thread's element in a pass
   for (int t0 = lo_t; t0 < hi_t; t0 += DT) {
     if (t0 + DT <= first) continue;             // (only the first pass of the first split can lie in front)
-    // scores of key t0 + tid with every head of the group; the key's pieces are asked for together, 16 at a time
-    const int t = t0 + tid;
-    const bool valid = t >= first && t <= pos;
-    float s[HG];
+    // ---- scores: 4 tiles of 16 keys a wave
+    {
+      Frag kf[4][KS];
 #pragma unroll
-    for (int j = 0; j < HG; ++j) s[j] = 0.f;
-    if (valid) {
-      const bf16_t* kp = head + (size_t)bt[t / P] * page_stride + (size_t)(t % P) * dk;
-      for (int c0 = 0; c0 < dk; c0 += FR * 8) {
-        Frag kf[FR];
+      for (int tt = 0; tt < 4; ++tt) {
+        const int t = t0 + wave * 64 + tt * 16 + li;
+        const bool seen = t >= first && t <= pos;
+        const bf16_t* kp = head + (size_t)(seen ? bt[t / P] : 0) * page_stride + (size_t)(t % P) * dk;
 #pragma unroll
-        for (int i = 0; i < FR; ++i)
-          if (c0 + i * 8 < dk) kf[i] = load_frag(kp + c0 + i * 8);
+        for (int ks = 0; ks < KS; ++ks) {
+          const int c = ks * 32 + lc * 8;
+          kf[tt][ks] = (seen && c < dk) ? load_frag(kp + c) : zero_frag();
+        }
+      }
 #pragma unroll
-        for (int i = 0; i < FR; ++i) {
-          if (c0 + i * 8 < dk) {
-            float kv[8];
+      for (int tt = 0; tt < 4; ++tt) {
+        floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-              kv[2 * w] = __uint_as_float(kf[i].w[w] << 16);
-              kv[2 * w + 1] = __uint_as_float(kf[i].w[w] & 0xffff0000u);
-            }
+        for (int ks = 0; ks < KS; ++ks) acc = mfma16(kf[tt][ks], qf[ks], acc);
+        // lane: keys tt * 16 + lc * 4 + 0..3 of the wave's 64, head li
+        *reinterpret_cast<float4*>(sc + li * SROW + wave * 64 + tt * 16 + lc * 4) =
+            float4{acc[0] * scale, acc[1] * scale, acc[2] * scale, acc[3] * scale};
+      }
+    }
+    // ---- this wave's value pieces are asked for now: they do not wait for the weights
+    Frag vf[ET][DT / 32];
 #pragma unroll
-            for (int j = 0; j < HG; ++j) {
-              if (j < per) {
-                const float4 qa = *reinterpret_cast<const float4*>(qs + j * DMAX + c0 + i * 8);
-                const float4 qb = *reinterpret_cast<const float4*>(qs + j * DMAX + c0 + i * 8 + 4);
-                float a = s[j];
-                a = fmaf(qa.x, kv[0], a); a = fmaf(qa.y, kv[1], a); a = fmaf(qa.z, kv[2], a); a = fmaf(qa.w, kv[3], a);
-                a = fmaf(qb.x, kv[4], a); a = fmaf(qb.y, kv[5], a); a = fmaf(qb.z, kv[6], a); a = fmaf(qb.w, kv[7], a);
-                s[j] = a;
-              }
-            }
+    for (int i = 0; i < ET; ++i) {
+      const int e = (wave + 4 * i) * 16 + li;
+      if (wave + 4 * i < n_et) {
+#pragma unroll
+        for (int kk = 0; kk < DT / 32; ++kk) {
+          const int tp = t0 + kk * 32 + lc * 8;
+          if (e < dv && tp <= pos && tp + 8 > first) {
+            vf[i][kk] = load_frag(head + (size_t)bt[tp / P] * page_stride + (size_t)P * dk + (size_t)e * P + tp % P);
+            if (tp < first || tp + 8 > pos + 1) keep_positions(vf[i][kk], first - tp, pos - tp + 1);
+          } else {
+            vf[i][kk] = zero_frag();
           }
         }
       }
     }
-    // the first pieces of the thread's value element are asked for now: they do not wait for the weights
-    // piece f of the thread: slots (sl + nsl * f) * 8 .. + 7 of the pass (a piece lies in one page)
-    Frag vf[FR];
-    auto piece_pos = [&](int f) { return t0 + (sl + nsl * f) * 8; };
-    auto load_values = [&](int f0) {
+    wave_lds_order();                           // the scores of keys 64 w .. are this wave's own
+    // ---- softmax, a key a thread
+    const int t = t0 + tid;
+    const bool valid = t >= first && t <= pos;
+    float s[HGMAX];
 #pragma unroll
-      for (int i = 0; i < FR; ++i) {
-        const int f = f0 + i;
-        if (f < nfr) {
-          const int tp = piece_pos(f);
-          if (tp <= pos && tp + 8 > first)
-            vf[i] = load_frag(head + (size_t)bt[tp / P] * page_stride + (size_t)P * dk + (size_t)e * P + tp % P);
-        }
-      }
-    };
-    if (e < dv) load_values(0);
-#pragma unroll
-    for (int j = 0; j < HG; ++j) {
+    for (int j = 0; j < HGMAX; ++j) {
       if (j < per) {
-        const float v = wave_max(valid ? s[j] : -INFINITY);
+        s[j] = valid ? sc[j * SROW + tid] : -INFINITY;
+        const float v = wave_max(s[j]);
         if (lane == 0) red[0][j][wave] = v;
       }
     }
-    __syncthreads();                            // (also: the pass before is done with ps)
-    float alpha[HG];
+    __syncthreads();                            // (also: the pass before is done with ps and al)
 #pragma unroll
-    for (int j = 0; j < HG; ++j) {
-      alpha[j] = 1.f;
+    for (int j = 0; j < HGMAX; ++j) {
       if (j < per) {
         float m_new = m_run[j];
 #pragma unroll
         for (int w = 0; w < DT / WAVE; ++w) m_new = fmaxf(m_new, red[0][j][w]);   // finite: the pass holds a key the row sees
-        alpha[j] = __expf(m_run[j] - m_new);
+        const float alpha = __expf(m_run[j] - m_new);
         m_run[j] = m_new;
         const float p = valid ? __expf(s[j] - m_new) : 0.f;
-        ps[j * DT + tid] = p;
+        ps[j * PROW + tid] = float_to_bf16(p);
         const float sum = wave_sum(p);
         if (lane == 0) red[1][j][wave] = sum;
+        if (tid == j) al[j] = alpha;
+        l_run[j] *= alpha;
       }
     }
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < HG; ++j) {
+    for (int j = 0; j < HGMAX; ++j) {
       if (j < per) {
-        float sum = 0.f;
 #pragma unroll
-        for (int w = 0; w < DT / WAVE; ++w) sum += red[1][j][w];
-        l_run[j] = l_run[j] * alpha[j] + sum;
-        o[j] *= alpha[j];
+        for (int w = 0; w < DT / WAVE; ++w) l_run[j] += red[1][j][w];
       }
     }
-    // values: element e at the thread's pieces of the pass
-    if (e < dv) {
-      for (int f0 = 0; f0 < nfr; f0 += FR) {
-        if (f0) load_values(f0);
+    // ---- values
+    const float my_alpha = li < per ? al[li] : 1.f;
+    Frag pf[DT / 32];
 #pragma unroll
-        for (int i = 0; i < FR; ++i) {
-          const int f = f0 + i;
-          if (f >= nfr) continue;
-          const int tp = piece_pos(f);
-          if (tp > pos || tp + 8 <= first) continue;
-          float vv[8];
+    for (int kk = 0; kk < DT / 32; ++kk) pf[kk] = *reinterpret_cast<const Frag*>(ps + li * PROW + kk * 32 + lc * 8);
 #pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            vv[2 * w] = __uint_as_float(vf[i].w[w] << 16);
-            vv[2 * w + 1] = __uint_as_float(vf[i].w[w] & 0xffff0000u);
-          }
+    for (int i = 0; i < ET; ++i) {
+      if (wave + 4 * i < n_et) {
 #pragma unroll
-          for (int k = 0; k < 8; ++k)             // slots the row does not see may hold anything
-            if (tp + k < first || tp + k > pos) vv[k] = 0.f;
-          const int k0 = tp - t0;
+        for (int rr = 0; rr < 4; ++rr) o[i][rr] *= my_alpha;
 #pragma unroll
-          for (int j = 0; j < HG; ++j) {
-            if (j < per) {
-              const float4 pa = *reinterpret_cast<const float4*>(ps + j * DT + k0);
-              const float4 pb = *reinterpret_cast<const float4*>(ps + j * DT + k0 + 4);
-              float a = o[j];
-              a = fmaf(pa.x, vv[0], a); a = fmaf(pa.y, vv[1], a); a = fmaf(pa.z, vv[2], a); a = fmaf(pa.w, vv[3], a);
-              a = fmaf(pb.x, vv[4], a); a = fmaf(pb.y, vv[5], a); a = fmaf(pb.z, vv[6], a); a = fmaf(pb.w, vv[7], a);
-              o[j] = a;
-            }
-          }
-        }
+        for (int kk = 0; kk < DT / 32; ++kk) o[i] = mfma16(vf[i][kk], pf[kk], o[i]);
       }
     }
   }
-  // the threads that share an element add up through LDS (qs is free now: every pass is behind a barrier)
-  __syncthreads();
-  float* acc = qs;                               // [HG][DT]: DT <= DMAX
+  // lane: elements (wave + 4 i) * 16 + lc * 4 + 0..3 of head li
+  if (li < per) {
+    float* p = parts + (((size_t)ri * H + g * per + li) * n_splits + split) * (dv + 2) + 2;
 #pragma unroll
-  for (int j = 0; j < HG; ++j)
-    if (j < per) acc[j * DMAX + tid] = o[j];
-  __syncthreads();
-  if (sl == 0 && e < dv) {
+    for (int i = 0; i < ET; ++i) {
 #pragma unroll
-    for (int j = 0; j < HG; ++j) {
-      if (j < per) {
-        float sum = 0.f;
-        for (int k = 0; k < nsl; ++k) sum += acc[j * DMAX + k * dvt + e];
-        parts[(((size_t)ri * H + g * per + j) * n_splits + split) * (dv + 2) + 2 + e] = sum;
+      for (int rr = 0; rr < 4; ++rr) {
+        const int e = (wave + 4 * i) * 16 + lc * 4 + rr;
+        if (wave + 4 * i < n_et && e < dv) p[e] = o[i][rr];
       }
     }
   }
@@ -450,7 +427,7 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     float* p = parts + (((size_t)ri * H + g * per + tid) * n_splits + split) * (dv + 2);
     float m = -INFINITY, l = 0.f;
 #pragma unroll
-    for (int j = 0; j < HG; ++j)
+    for (int j = 0; j < HGMAX; ++j)
       if (j == tid) { m = m_run[j]; l = l_run[j]; }
     p[0] = m;
     p[1] = l;
@@ -550,16 +527,20 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
       (long)n_rows * G * n_splits > 0x7fffffffL || H > 65535)
     return APC_ERR_BAD_ARG;
   dim3 grid(n_rows * G * n_splits), block(DT);
-  const int per = H / G;
-#define MD_LAUNCH(HG_)                                                                                              \
-  hipLaunchKernelGGL((attn_masked_decode_kernel<HG_>), grid, block, 0, stream, (const bf16_t*)q, ldq, H, G, dk, dv, \
-                     (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg, rows, mask,     \
+#define MD_LAUNCH(KS_, ET_)                                                                                       \
+  hipLaunchKernelGGL((attn_masked_decode_kernel<KS_, ET_>), grid, block, 0, stream, (const bf16_t*)q, ldq, H, G, dk, \
+                     dv, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg, rows, mask,  \
                      mask_size, scale, n_splits, keys_per_split, parts)
-  if (per <= 1) MD_LAUNCH(1);
-  else if (per <= 2) MD_LAUNCH(2);
-  else if (per <= 4) MD_LAUNCH(4);
-  else if (per <= 8) MD_LAUNCH(8);
-  else MD_LAUNCH(16);
+#define MD_VALUES(KS_)                    \
+  do {                                    \
+    if (dv <= 64) MD_LAUNCH(KS_, 1);      \
+    else if (dv <= 128) MD_LAUNCH(KS_, 2); \
+    else MD_LAUNCH(KS_, 4);               \
+  } while (0)
+  if (dk <= 64) MD_VALUES(2);
+  else if (dk <= 128) MD_VALUES(4);
+  else MD_VALUES(8);
+#undef MD_VALUES
 #undef MD_LAUNCH
   APC_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn_masked_merge_kernel, dim3(n_rows, H), dim3(64), 0, stream, parts, n_splits, H, dv, rows, sink,

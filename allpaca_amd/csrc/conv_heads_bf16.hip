@@ -1,5 +1,5 @@
 // The short convolution on the heads of projected rows (see plain_mixers.hip for the formulas) for bfloat16 rows, 16
-// bytes a thread: a block takes ROWS consecutive rows whole, a thread PPT pieces of 8 channels of each, with the taps of
+// bytes a thread: a block takes ROWS (2 or 4) consecutive rows whole, a thread PPT pieces of 8 channels of each, with the taps of
 // its channels in registers.  Sums of squares of the pieces go through LDS, so a head may be any multiple of 8 wide.
 // The row holds q heads, then k heads, then v heads.  The state of the convolution is moved on by the plain kernel.
 #include "mfma.h"
@@ -8,7 +8,6 @@
 namespace {
 
 constexpr int MAXT = 4;   // taps
-constexpr int ROWS = 2;
 
 __device__ __forceinline__ void unpack8(const Frag& f, float* v) {
 #pragma unroll
@@ -18,14 +17,15 @@ __device__ __forceinline__ void unpack8(const Frag& f, float* v) {
   }
 }
 
-template <int PPT>
+template <int PPT, int ROWS, int TAPS>
 __global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
     const bf16_t* __restrict__ proj, int ld, int n_rows, int H, int G, int dk, int dv, const float* __restrict__ bias,
-    const float* __restrict__ conv_w, int taps, const float* __restrict__ state, int width,
+    const float* __restrict__ conv_w, const float* __restrict__ state, int width,
     const int* __restrict__ row_seg, const int* __restrict__ seg_row0, const int* __restrict__ slots,
     const int* __restrict__ positions, int unit_norm, float eps, bf16_t* __restrict__ q_out, int ldq,
     const int* __restrict__ block_table, int max_blocks, bf16_t* __restrict__ cache, int P) {
   extern __shared__ float ssum[];            // [ROWS][pieces]
+  constexpr int taps = TAPS;
   const int tid = threadIdx.x;
   const int pieces = width / 8;
   const int r0 = blockIdx.x * ROWS;
@@ -44,15 +44,19 @@ __global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
     const int p = tid + 256 * k;
     if (p >= pieces) continue;
     const int c0 = p * 8;
-    float b[8], w[8 * MAXT];
+    float b[8], w[8 * TAPS];                         // w[e * TAPS + j], as the taps lie in memory
 #pragma unroll
-    for (int e = 0; e < 8; ++e) b[e] = bias ? bias[c0 + e] : 0.f;
-    if (taps > 1) {
+    for (int e = 0; e < 8; ++e) b[e] = 0.f;
+    if (bias) {
+      const float4 a = *reinterpret_cast<const float4*>(bias + c0), c = *reinterpret_cast<const float4*>(bias + c0 + 4);
+      b[0] = a.x; b[1] = a.y; b[2] = a.z; b[3] = a.w; b[4] = c.x; b[5] = c.y; b[6] = c.z; b[7] = c.w;
+    }
+    if (TAPS > 1) {
 #pragma unroll
-      for (int j = 0; j < MAXT; ++j)
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (j < taps) w[j * 8 + e] = conv_w[(size_t)(c0 + e) * taps + j];
+      for (int i = 0; i < 2 * TAPS; ++i) {
+        const float4 a = *reinterpret_cast<const float4*>(conv_w + (size_t)c0 * TAPS + 4 * i);
+        w[4 * i] = a.x; w[4 * i + 1] = a.y; w[4 * i + 2] = a.z; w[4 * i + 3] = a.w;
+      }
     }
 #pragma unroll
     for (int rr = 0; rr < ROWS; ++rr) {
@@ -61,8 +65,8 @@ __global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] = 0.f;
 #pragma unroll
-      for (int j = 0; j < MAXT; ++j) {                 // oldest first, as the plain kernel adds
-        if (j < taps) {
+      for (int j = 0; j < TAPS; ++j) {                 // oldest first, as the plain kernel adds
+        {
           const int back = taps - 1 - j;
           float u[8];
           if (back <= in_seg[rr]) {
@@ -76,7 +80,7 @@ __global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
           }
           if (taps > 1) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] = fmaf(w[j * 8 + e], u[e], acc[e]);
+            for (int e = 0; e < 8; ++e) acc[e] = fmaf(w[e * TAPS + j], u[e], acc[e]);
           } else {
 #pragma unroll
             for (int e = 0; e < 8; ++e) acc[e] = u[e];
@@ -148,22 +152,32 @@ APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, 
                                    int page_tokens, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (!apc_conv_heads_bf16_takes(ld, width, H, G, dk, dv, taps, ldq)) return APC_ERR_UNSUPPORTED;
-  if (((uintptr_t)proj & 15u) || ((uintptr_t)q_out & 15u) || ((uintptr_t)cache & 15u) || ((uintptr_t)state & 15u))
+  if (((uintptr_t)proj & 15u) || ((uintptr_t)q_out & 15u) || ((uintptr_t)cache & 15u) || ((uintptr_t)state & 15u) ||
+      ((uintptr_t)bias & 15u) || ((uintptr_t)conv_w & 15u))
     return APC_ERR_UNSUPPORTED;
   if (taps > 1 && (!conv_w || !state || !slots)) return APC_ERR_BAD_ARG;
   if (G > 0 && (!cache || !block_table || page_tokens <= 0 || max_blocks <= 0)) return APC_ERR_BAD_ARG;
   const int pieces = width / 8;
   const int ppt = (pieces + 255) / 256;
-  dim3 grid((n_rows + ROWS - 1) / ROWS), block(256);
-  const size_t lds = (size_t)ROWS * pieces * sizeof(float);
-#define CH_LAUNCH(PPT_)                                                                                               \
-  hipLaunchKernelGGL((conv_heads_bf16_kernel<PPT_>), grid, block, lds, stream, (const bf16_t*)proj, ld, n_rows, H, G, \
-                     dk, dv, bias, conv_w, taps, state, width, row_seg, seg_row0, slots, positions, unit_norm, eps,    \
-                     (bf16_t*)q_out, ldq, block_table, max_blocks, (bf16_t*)cache, page_tokens)
-  if (ppt <= 1) CH_LAUNCH(1);
-  else if (ppt <= 2) CH_LAUNCH(2);
-  else if (ppt <= 4) CH_LAUNCH(4);
-  else CH_LAUNCH(8);
+  const int rows_a_block = ppt <= 2 ? 4 : 2;   // (a thread keeps its channels' taps for all rows of the block)
+  dim3 grid((n_rows + rows_a_block - 1) / rows_a_block), block(256);
+  const size_t lds = (size_t)rows_a_block * pieces * sizeof(float);
+#define CH_LAUNCH(PPT_, ROWS_, TAPS_)                                                                              \
+  hipLaunchKernelGGL((conv_heads_bf16_kernel<PPT_, ROWS_, TAPS_>), grid, block, lds, stream, (const bf16_t*)proj,  \
+                     ld, n_rows, H, G, dk, dv, bias, conv_w, state, width, row_seg, seg_row0, slots, positions,     \
+                     unit_norm, eps, (bf16_t*)q_out, ldq, block_table, max_blocks, (bf16_t*)cache, page_tokens)
+#define CH_TAPS(PPT_, ROWS_)                            \
+  do {                                                  \
+    if (taps == 1) CH_LAUNCH(PPT_, ROWS_, 1);           \
+    else if (taps == 2) CH_LAUNCH(PPT_, ROWS_, 2);      \
+    else if (taps == 3) CH_LAUNCH(PPT_, ROWS_, 3);      \
+    else CH_LAUNCH(PPT_, ROWS_, 4);                     \
+  } while (0)
+  if (ppt <= 1) CH_TAPS(1, 4);
+  else if (ppt <= 2) CH_TAPS(2, 4);
+  else if (ppt <= 4) CH_TAPS(4, 2);
+  else CH_TAPS(8, 2);
+#undef CH_TAPS
 #undef CH_LAUNCH
   APC_LAUNCH_CHECK();
   return 0;
