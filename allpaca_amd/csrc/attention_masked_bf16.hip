@@ -259,33 +259,36 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
 }
 
 // ------------------------------------------------------------------------------------------ decoded rows
-constexpr int DT = 256;       // keys of a pass: one a thread in the softmax
+constexpr int DT = 256;       // keys of a block's pass: 64 a wave
 constexpr int DMAX = 256;     // largest key and value size
 constexpr int HGMAX = 16;     // query heads of a kv head: the 16 columns of an MFMA tile
-constexpr int SROW = DT + 4;  // floats of a row of scores in LDS (heads then fall into different banks)
-constexpr int PROW = DT + 8;  // bfloat16 of a row of weights in LDS
+constexpr int SROW = 64 + 4;  // floats of a row of a wave's scores in LDS (heads then fall into different banks)
+constexpr int PROW = 64 + 8;  // bfloat16 of a row of a wave's weights in LDS
+constexpr int NW = DT / WAVE;
 
-// grid: rows x G x n_splits.  Split s of a row takes the keys at positions a0 + s * kps .. a0 + (s + 1) * kps - 1 that
-// the row sees, a0 being the row's first key rounded down to a multiple of DT (kps is a multiple of DT, pages are
-// powers of two up to DT: 8 consecutive positions from a multiple of 8 on lie in one page).  It leaves, per query head
-// of the group, the maximum score m, sum exp(s - m) and sum exp(s - m) v of its keys in `parts`
-// [row][head][split][2 + dv].
-// A pass of 256 keys: wave w forms the scores of keys 64 w .. 64 w + 63 with all heads of the group (S = K Q^T, keys
-// as the rows of the tile, straight from the pages), the block takes maxima and sums with a key a thread, the weights go
-// to LDS in bfloat16, and wave w adds up value elements 16 (w + 4 i) .. + 15 over all 256 keys (O^T = V^T P^T, 8 slots of
-// an element a lane, straight from the pages).
-template <int KS, int ET>  // 32-element steps over a key; value tiles of 16 elements a wave
+// grid: rows x G x n_splits, 4 waves a block.  Split s of a row takes the keys at positions a0 + s * kps ..
+// a0 + (s + 1) * kps - 1 that the row sees, a0 being the row's first key rounded down to a multiple of 256 (kps is a
+// multiple of 256; pages are powers of two up to 256, so 8 consecutive positions from a multiple of 8 on lie in one
+// page); of every 256 of them wave w takes keys 64 w .. 64 w + 63.  A wave is a part of its own: it leaves, per query
+// head of the group, the maximum score m, sum exp(s - m) and sum exp(s - m) v of its keys in `parts`
+// [row][head][4 s + w][2 + dv], and no wave waits for another.
+// 64 keys: scores with all heads of the group as S = K Q^T (keys as the rows of 4 tiles, straight from the pages into
+// the operand), maxima and sums with a key a lane, weights to LDS in bfloat16, then O^T += V^T P^T over the 64 keys for
+// every 16 value elements (8 slots of an element a lane, straight from the pages).
+template <int KS, int ET>  // 32-element steps over a key; tiles of 16 value elements
 __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     const bf16_t* __restrict__ q, int ldq, int H, int G, int dk, int dv, const bf16_t* __restrict__ cache, int P,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ positions,
     const int* __restrict__ row_seg, const int* __restrict__ rows, int mask, int mask_size, float scale, int n_splits,
     int kps, float* __restrict__ parts) {
-  __shared__ __attribute__((aligned(16))) float sc[HGMAX * SROW];
-  __shared__ __attribute__((aligned(16))) bf16_t ps[HGMAX * PROW];
-  __shared__ float red[2][HGMAX][DT / WAVE];
-  __shared__ float al[HGMAX];
+  __shared__ __attribute__((aligned(16))) float sc_all[NW][HGMAX * SROW];
+  __shared__ __attribute__((aligned(16))) bf16_t ps_all[NW][HGMAX * PROW];
+  __shared__ float ml_all[NW][HGMAX][3];        // running maximum, running sum, the last pass's factor
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const int li = lane % 16, lc = lane / 16;
+  float* sc = sc_all[wave];
+  bf16_t* ps = ps_all[wave];
+  float(*ml)[3] = ml_all[wave];
   const int split = blockIdx.x % n_splits, g = (blockIdx.x / n_splits) % G, ri = blockIdx.x / (n_splits * G);
   const int r = rows ? rows[ri] : ri;
   const int per = H / G;                        // query heads of this kv head (<= HGMAX)
@@ -303,25 +306,23 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     const int c = ks * 32 + lc * 8;
     qf[ks] = (li < per && c < dk) ? load_frag(q + (size_t)r * ldq + (size_t)(g * per + li) * dk + c) : zero_frag();
   }
-  for (int idx = tid; idx < HGMAX * PROW; idx += DT) ps[idx] = 0;    // rows of heads that do not exist stay 0
-  float m_run[HGMAX], l_run[HGMAX];
-#pragma unroll
-  for (int j = 0; j < HGMAX; ++j) { m_run[j] = -INFINITY; l_run[j] = 0.f; }
+  for (int idx = lane; idx < HGMAX * PROW; idx += WAVE) ps[idx] = 0;    // rows of heads that do not exist stay 0
+  if (lane < HGMAX) { ml[lane][0] = -INFINITY; ml[lane][1] = 0.f; ml[lane][2] = 1.f; }
   floatx4 o[ET];
 #pragma unroll
   for (int i = 0; i < ET; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const int n_et = (dv + 15) / 16;
+  wave_lds_order();
 
   const int lo_t = a0 + split * kps;
   const int hi_t = min(lo_t + kps, pos + 1);
-  for (int t0 = lo_t; t0 < hi_t; t0 += DT) {
-    if (t0 + DT <= first) continue;             // (only the first pass of the first split can lie in front)
-    // ---- scores: 4 tiles of 16 keys a wave
+  for (int t0 = lo_t + wave * WAVE; t0 < hi_t; t0 += DT) {
+    if (t0 + WAVE <= first) continue;           // (only in front of the row's first key)
+    // ---- scores of keys t0 .. t0 + 63: 4 tiles of 16 keys
     {
       Frag kf[4][KS];
 #pragma unroll
       for (int tt = 0; tt < 4; ++tt) {
-        const int t = t0 + wave * 64 + tt * 16 + li;
+        const int t = t0 + tt * 16 + li;
         const bool seen = t >= first && t <= pos;
         const bf16_t* kp = head + (size_t)(seen ? bt[t / P] : 0) * page_stride + (size_t)(t % P) * dk;
 #pragma unroll
@@ -335,127 +336,97 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
         floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) acc = mfma16(kf[tt][ks], qf[ks], acc);
-        // lane: keys tt * 16 + lc * 4 + 0..3 of the wave's 64, head li
-        *reinterpret_cast<float4*>(sc + li * SROW + wave * 64 + tt * 16 + lc * 4) =
+        // lane: keys tt * 16 + lc * 4 + 0..3 of the 64, head li
+        *reinterpret_cast<float4*>(sc + li * SROW + tt * 16 + lc * 4) =
             float4{acc[0] * scale, acc[1] * scale, acc[2] * scale, acc[3] * scale};
       }
     }
-    // ---- this wave's value pieces are asked for now: they do not wait for the weights
-    Frag vf[ET][DT / 32];
+    // ---- the value pieces are asked for now: they do not wait for the weights
+    Frag vf[ET][2];
 #pragma unroll
     for (int i = 0; i < ET; ++i) {
-      const int e = (wave + 4 * i) * 16 + li;
-      if (wave + 4 * i < n_et) {
+      const int e = i * 16 + li;
 #pragma unroll
-        for (int kk = 0; kk < DT / 32; ++kk) {
-          const int tp = t0 + kk * 32 + lc * 8;
-          if (e < dv && tp <= pos && tp + 8 > first) {
-            vf[i][kk] = load_frag(head + (size_t)bt[tp / P] * page_stride + (size_t)P * dk + (size_t)e * P + tp % P);
-            if (tp < first || tp + 8 > pos + 1) keep_positions(vf[i][kk], first - tp, pos - tp + 1);
-          } else {
-            vf[i][kk] = zero_frag();
-          }
+      for (int kk = 0; kk < 2; ++kk) {
+        const int tp = t0 + kk * 32 + lc * 8;
+        if (e < dv && tp <= pos && tp + 8 > first) {
+          vf[i][kk] = load_frag(head + (size_t)bt[tp / P] * page_stride + (size_t)P * dk + (size_t)e * P + tp % P);
+          if (tp < first || tp + 8 > pos + 1) keep_positions(vf[i][kk], first - tp, pos - tp + 1);
+        } else {
+          vf[i][kk] = zero_frag();
         }
       }
     }
-    wave_lds_order();                           // the scores of keys 64 w .. are this wave's own
-    // ---- softmax, a key a thread
-    const int t = t0 + tid;
+    wave_lds_order();
+    // ---- softmax, a key a lane
+    const int t = t0 + lane;
     const bool valid = t >= first && t <= pos;
-    float s[HGMAX];
-#pragma unroll
-    for (int j = 0; j < HGMAX; ++j) {
-      if (j < per) {
-        s[j] = valid ? sc[j * SROW + tid] : -INFINITY;
-        const float v = wave_max(s[j]);
-        if (lane == 0) red[0][j][wave] = v;
-      }
+    for (int j = 0; j < per; ++j) {
+      const float s = valid ? sc[j * SROW + lane] : -INFINITY;
+      const float m_old = ml[j][0], l_old = ml[j][1];
+      const float m_new = fmaxf(m_old, wave_max(s));   // finite: the 64 keys hold one the row sees
+      const float alpha = __expf(m_old - m_new);
+      const float p = valid ? __expf(s - m_new) : 0.f;
+      ps[j * PROW + lane] = float_to_bf16(p);
+      const float l_new = l_old * alpha + wave_sum(p);
+      wave_lds_order();                           // every lane has read the old values
+      if (lane == 0) { ml[j][0] = m_new; ml[j][1] = l_new; ml[j][2] = alpha; }
     }
-    __syncthreads();                            // (also: the pass before is done with ps and al)
-#pragma unroll
-    for (int j = 0; j < HGMAX; ++j) {
-      if (j < per) {
-        float m_new = m_run[j];
-#pragma unroll
-        for (int w = 0; w < DT / WAVE; ++w) m_new = fmaxf(m_new, red[0][j][w]);   // finite: the pass holds a key the row sees
-        const float alpha = __expf(m_run[j] - m_new);
-        m_run[j] = m_new;
-        const float p = valid ? __expf(s[j] - m_new) : 0.f;
-        ps[j * PROW + tid] = float_to_bf16(p);
-        const float sum = wave_sum(p);
-        if (lane == 0) red[1][j][wave] = sum;
-        if (tid == j) al[j] = alpha;
-        l_run[j] *= alpha;
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < HGMAX; ++j) {
-      if (j < per) {
-#pragma unroll
-        for (int w = 0; w < DT / WAVE; ++w) l_run[j] += red[1][j][w];
-      }
-    }
+    wave_lds_order();
     // ---- values
-    const float my_alpha = li < per ? al[li] : 1.f;
-    Frag pf[DT / 32];
+    const float my_alpha = li < per ? ml[li][2] : 1.f;
+    Frag pf[2];
 #pragma unroll
-    for (int kk = 0; kk < DT / 32; ++kk) pf[kk] = *reinterpret_cast<const Frag*>(ps + li * PROW + kk * 32 + lc * 8);
+    for (int kk = 0; kk < 2; ++kk) pf[kk] = *reinterpret_cast<const Frag*>(ps + li * PROW + kk * 32 + lc * 8);
 #pragma unroll
     for (int i = 0; i < ET; ++i) {
-      if (wave + 4 * i < n_et) {
 #pragma unroll
-        for (int rr = 0; rr < 4; ++rr) o[i][rr] *= my_alpha;
+      for (int rr = 0; rr < 4; ++rr) o[i][rr] *= my_alpha;
 #pragma unroll
-        for (int kk = 0; kk < DT / 32; ++kk) o[i] = mfma16(vf[i][kk], pf[kk], o[i]);
-      }
+      for (int kk = 0; kk < 2; ++kk) o[i] = mfma16(vf[i][kk], pf[kk], o[i]);
     }
+    wave_lds_order();
   }
-  // lane: elements (wave + 4 i) * 16 + lc * 4 + 0..3 of head li
+  // lane: elements i * 16 + lc * 4 + 0..3 of head li
+  const int n_parts = n_splits * NW, part = split * NW + wave;
   if (li < per) {
-    float* p = parts + (((size_t)ri * H + g * per + li) * n_splits + split) * (dv + 2) + 2;
+    float* p = parts + (((size_t)ri * H + g * per + li) * n_parts + part) * (dv + 2);
 #pragma unroll
     for (int i = 0; i < ET; ++i) {
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
-        const int e = (wave + 4 * i) * 16 + lc * 4 + rr;
-        if (wave + 4 * i < n_et && e < dv) p[e] = o[i][rr];
+        const int e = i * 16 + lc * 4 + rr;
+        if (e < dv) p[2 + e] = o[i][rr];
       }
     }
-  }
-  if (tid < per) {
-    float* p = parts + (((size_t)ri * H + g * per + tid) * n_splits + split) * (dv + 2);
-    float m = -INFINITY, l = 0.f;
-#pragma unroll
-    for (int j = 0; j < HGMAX; ++j)
-      if (j == tid) { m = m_run[j]; l = l_run[j]; }
-    p[0] = m;
-    p[1] = l;
+    if (lc == 0) { p[0] = ml[li][0]; p[1] = ml[li][1]; }
   }
 }
 
-// out[row][head] = sum_s e^(m_s - M) o_s / (sink e^(-M) + sum_s e^(m_s - M) l_s),  M = max(m_s, 0 with a sink)
-__global__ __launch_bounds__(64) void attn_masked_merge_kernel(const float* __restrict__ parts, int n_splits, int H,
+// out[row][head] = sum_s e^(m_s - M) o_s / (sink e^(-M) + sum_s e^(m_s - M) l_s),  M = max(m_s, 0 with a sink);
+// at most 64 parts: lane s holds part s's maximum and sum
+__global__ __launch_bounds__(64) void attn_masked_merge_kernel(const float* __restrict__ parts, int n_parts, int H,
                                                                int dv, const int* __restrict__ rows, int sink,
                                                                bf16_t* __restrict__ out, int ldo) {
   const int ri = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = rows ? rows[ri] : ri;
-  const float* p = parts + ((size_t)ri * H + h) * n_splits * (dv + 2);
-  float M = sink ? 0.f : -INFINITY;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, p[(size_t)s * (dv + 2)]);
-  float L = sink ? __expf(-M) : 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float m = p[(size_t)s * (dv + 2)];
-    if (m != -INFINITY) L += __expf(m - M) * p[(size_t)s * (dv + 2) + 1];
-  }
+  const float* p = parts + ((size_t)ri * H + h) * n_parts * (dv + 2);
+  const float m = lane < n_parts ? p[(size_t)lane * (dv + 2)] : -INFINITY;
+  const float l = lane < n_parts ? p[(size_t)lane * (dv + 2) + 1] : 0.f;
+  float M = wave_max(m);
+  if (sink) M = fmaxf(M, 0.f);
+  const float w = m == -INFINITY ? 0.f : __expf(m - M);
+  const float L = wave_sum(w * l) + (sink ? __expf(-M) : 0.f);
   const float inv = 1.0f / L;
-  for (int e = lane; e < dv; e += WAVE) {
+  for (int e0 = 0; e0 < dv; e0 += WAVE) {
+    const int e = e0 + lane;
     float a = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float m = p[(size_t)s * (dv + 2)];
-      if (m != -INFINITY) a = fmaf(__expf(m - M), p[(size_t)s * (dv + 2) + 2 + e], a);
+#pragma unroll 4
+    for (int s = 0; s < n_parts; ++s) {
+      const float ws = __shfl(w, s, WAVE);
+      if (e < dv) a = fmaf(ws, p[(size_t)s * (dv + 2) + 2 + e], a);
     }
-    out[(size_t)r * ldo + (size_t)h * dv + e] = float_to_bf16(a * inv);
+    if (e < dv) out[(size_t)r * ldo + (size_t)h * dv + e] = float_to_bf16(a * inv);
   }
 }
 
@@ -512,7 +483,7 @@ APC_EXPORT int apc_attention_masked_prefill_bf16(const void* q, int ldq, void* o
 }
 
 // `rows`: the step's rows that are decoded ones (nullptr: all n_rows rows); `keys_per_split`: a multiple of 256;
-// `parts`: room for n_rows * H * n_splits * (dv + 2) floats.
+// at most 16 splits; `parts`: room for n_rows * H * 4 * n_splits * (dv + 2) floats.
 APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* out, int ldo, int n_rows, int H, int G,
                                                 int dk, int dv, const void* cache, int page_tokens,
                                                 const int* block_table, int max_blocks, const int* positions,
@@ -523,7 +494,7 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
   int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale);
   if (e) return e;
   if (!apc_attention_masked_takes(H, G, dk, dv, page_tokens)) return APC_ERR_UNSUPPORTED;
-  if (n_splits <= 0 || keys_per_split <= 0 || keys_per_split % DT || !parts || max_blocks <= 0 ||
+  if (n_splits <= 0 || n_splits * NW > WAVE || keys_per_split <= 0 || keys_per_split % DT || !parts || max_blocks <= 0 ||
       (long)n_rows * G * n_splits > 0x7fffffffL || H > 65535)
     return APC_ERR_BAD_ARG;
   dim3 grid(n_rows * G * n_splits), block(DT);
@@ -531,11 +502,11 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
   hipLaunchKernelGGL((attn_masked_decode_kernel<KS_, ET_>), grid, block, 0, stream, (const bf16_t*)q, ldq, H, G, dk, \
                      dv, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg, rows, mask,  \
                      mask_size, scale, n_splits, keys_per_split, parts)
-#define MD_VALUES(KS_)                    \
-  do {                                    \
-    if (dv <= 64) MD_LAUNCH(KS_, 1);      \
-    else if (dv <= 128) MD_LAUNCH(KS_, 2); \
-    else MD_LAUNCH(KS_, 4);               \
+#define MD_VALUES(KS_)                     \
+  do {                                     \
+    if (dv <= 64) MD_LAUNCH(KS_, 4);       \
+    else if (dv <= 128) MD_LAUNCH(KS_, 8); \
+    else MD_LAUNCH(KS_, 16);               \
   } while (0)
   if (dk <= 64) MD_VALUES(2);
   else if (dk <= 128) MD_VALUES(4);
@@ -543,7 +514,7 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
 #undef MD_VALUES
 #undef MD_LAUNCH
   APC_LAUNCH_CHECK();
-  hipLaunchKernelGGL(attn_masked_merge_kernel, dim3(n_rows, H), dim3(64), 0, stream, parts, n_splits, H, dv, rows, sink,
+  hipLaunchKernelGGL(attn_masked_merge_kernel, dim3(n_rows, H), dim3(64), 0, stream, parts, n_splits * NW, H, dv, rows, sink,
                      (bf16_t*)out, ldo);
   APC_LAUNCH_CHECK();
   return 0;

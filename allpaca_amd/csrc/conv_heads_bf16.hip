@@ -38,6 +38,9 @@ __global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
     in_seg[rr] = r - seg_row0[seg[rr]];
     st[rr] = taps > 1 ? state + (size_t)slots[seg[rr]] * (taps - 1) * width : nullptr;
   }
+  bool block_all_in = r0 >= TAPS - 1;
+#pragma unroll
+  for (int rr = 0; rr < ROWS; ++rr) block_all_in = block_all_in && in_seg[rr] >= TAPS - 1;
   float y[PPT][ROWS][8];
 #pragma unroll
   for (int k = 0; k < PPT; ++k) {
@@ -58,39 +61,71 @@ __global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
         w[4 * i] = a.x; w[4 * i + 1] = a.y; w[4 * i + 2] = a.z; w[4 * i + 3] = a.w;
       }
     }
+    // The rows' inputs are asked for together and used afterwards, so the loads are in flight at once.  When every row
+    // of the block has its TAPS - 1 predecessors in its own segment (all but the first rows of a prompt portion), the
+    // ROWS + TAPS - 1 rows from r0 - (TAPS - 1) on serve all of them.
+    if (block_all_in) {
+      Frag src[ROWS + TAPS - 1];
 #pragma unroll
-    for (int rr = 0; rr < ROWS; ++rr) {
-      const int r = min(r0 + rr, n_rows - 1);
-      float acc[8];
+      for (int i = 0; i < ROWS + TAPS - 1; ++i)
+        src[i] = load_frag(proj + (size_t)min(r0 - (TAPS - 1) + i, n_rows - 1) * ld + c0);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+      for (int rr = 0; rr < ROWS; ++rr) {
+        float acc[8];
 #pragma unroll
-      for (int j = 0; j < TAPS; ++j) {                 // oldest first, as the plain kernel adds
-        {
-          const int back = taps - 1 - j;
+        for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {               // oldest first, as the plain kernel adds
+          float u[8];
+          unpack8(src[rr + j], u);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] = TAPS > 1 ? fmaf(w[e * TAPS + j], u[e] + b[e], acc[e]) : u[e] + b[e];
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { y[k][rr][e] = acc[e]; ss = fmaf(acc[e], acc[e], ss); }
+        ssum[rr * pieces + p] = ss;
+      }
+    } else {
+#pragma unroll
+      for (int rr = 0; rr < ROWS; ++rr) {
+        const int r = min(r0 + rr, n_rows - 1);
+        Frag raw[TAPS];
+        float4 sa[TAPS], sb[TAPS];
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {
+          const int back = TAPS - 1 - j;
+          if (back <= in_seg[rr]) {
+            raw[j] = load_frag(proj + (size_t)(r - back) * ld + c0);
+          } else {
+            const float* sp = st[rr] + (size_t)(TAPS - 1 - (back - in_seg[rr])) * width + c0;
+            sa[j] = *reinterpret_cast<const float4*>(sp);
+            sb[j] = *reinterpret_cast<const float4*>(sp + 4);
+          }
+        }
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {
+          const int back = TAPS - 1 - j;
           float u[8];
           if (back <= in_seg[rr]) {
-            unpack8(load_frag(proj + (size_t)(r - back) * ld + c0), u);
+            unpack8(raw[j], u);
 #pragma unroll
             for (int e = 0; e < 8; ++e) u[e] += b[e];
           } else {
-            const float* sp = st[rr] + (size_t)(taps - 1 - (back - in_seg[rr])) * width + c0;
-            const float4 a = *reinterpret_cast<const float4*>(sp), c = *reinterpret_cast<const float4*>(sp + 4);
-            u[0] = a.x; u[1] = a.y; u[2] = a.z; u[3] = a.w; u[4] = c.x; u[5] = c.y; u[6] = c.z; u[7] = c.w;
+            u[0] = sa[j].x; u[1] = sa[j].y; u[2] = sa[j].z; u[3] = sa[j].w;
+            u[4] = sb[j].x; u[5] = sb[j].y; u[6] = sb[j].z; u[7] = sb[j].w;
           }
-          if (taps > 1) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] = fmaf(w[e * TAPS + j], u[e], acc[e]);
-          } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] = u[e];
-          }
+          for (int e = 0; e < 8; ++e) acc[e] = TAPS > 1 ? fmaf(w[e * TAPS + j], u[e], acc[e]) : u[e];
         }
-      }
-      float ss = 0.f;
+        float ss = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { y[k][rr][e] = acc[e]; ss = fmaf(acc[e], acc[e], ss); }
-      ssum[rr * pieces + p] = ss;
+        for (int e = 0; e < 8; ++e) { y[k][rr][e] = acc[e]; ss = fmaf(acc[e], acc[e], ss); }
+        ssum[rr * pieces + p] = ss;
+      }
     }
   }
   __syncthreads();
@@ -159,7 +194,7 @@ APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, 
   if (G > 0 && (!cache || !block_table || page_tokens <= 0 || max_blocks <= 0)) return APC_ERR_BAD_ARG;
   const int pieces = width / 8;
   const int ppt = (pieces + 255) / 256;
-  const int rows_a_block = ppt <= 2 ? 4 : 2;   // (a thread keeps its channels' taps for all rows of the block)
+  const int rows_a_block = ppt <= 4 ? 4 : 2;   // (a thread keeps its channels' taps for all rows of the block)
   dim3 grid((n_rows + rows_a_block - 1) / rows_a_block), block(256);
   const size_t lds = (size_t)rows_a_block * pieces * sizeof(float);
 #define CH_LAUNCH(PPT_, ROWS_, TAPS_)                                                                              \
@@ -175,7 +210,7 @@ APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, 
   } while (0)
   if (ppt <= 1) CH_TAPS(1, 4);
   else if (ppt <= 2) CH_TAPS(2, 4);
-  else if (ppt <= 4) CH_TAPS(4, 2);
+  else if (ppt <= 4) CH_TAPS(4, 4);
   else CH_TAPS(8, 2);
 #undef CH_TAPS
 #undef CH_LAUNCH

@@ -437,7 +437,7 @@ def sampler_times(vocab: int) -> dict:
 DESIGN_SIZES = {"1b": (2048, 32, 8, 64, 8192, 128256), "8b": (4096, 32, 8, 128, 14336, 128256)}
 # entry points of the new design -> the like entry points of the llama decoder
 LIKE_KERNELS = {
-    "apc_conv_heads": ["apc_rope_kv_write_bf16", "apc_rope_kv_write"],
+    "apc_conv_heads_bf16": ["apc_rope_kv_write_bf16", "apc_rope_kv_write"],
     "apc_attention_masked_prefill_bf16": ["apc_attention_prefill_bf16"],
     "apc_attention_masked_decode_bf16": ["apc_attention_decode_bf16"],
     "apc_streams_step": ["apc_rmsnorm_rows"],
@@ -539,7 +539,7 @@ def design_rooflines(size, layers, streams, batch, context, T, points):
 
     def work(name, rows, keys_sum):
         """(bytes, flops) of all of a step's launches of entry point `name`."""
-        if name in ("apc_conv_heads", "apc_rope_kv_write_bf16", "apc_rope_kv_write"):
+        if name in ("apc_conv_heads_bf16", "apc_rope_kv_write_bf16", "apc_rope_kv_write"):
             return layers * rows * (qkv + H * d + 2 * G * d) * 2, 0       # rows read, q and the pages' rows written
         if name in ("apc_attention_masked_prefill_bf16", "apc_attention_prefill_bf16"):
             return 0, layers * 4 * keys_sum * H * d

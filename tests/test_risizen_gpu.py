@@ -213,7 +213,7 @@ def test_clamped_glu_and_embedding_into_streams(dtype):
     from allpaca_amd.kernels import ops
     rng = np.random.default_rng(3)
     tdt = DTYPES[dtype]
-    T, D, F, limit = 5, 24, 50, 0.8
+    T, D, F, limit = 5, 24, (50 if dtype == "float32" else 56), 0.8      # (56: the kernel of 16-byte loads)
     h = torch.as_tensor(rng.normal(size=(T, D)), dtype=torch.float32).to(tdt)
     wg = torch.as_tensor(rng.normal(size=(F, D)), dtype=torch.float32).to(tdt)
     wu = torch.as_tensor(rng.normal(size=(F, D)), dtype=torch.float32).to(tdt)
@@ -221,6 +221,12 @@ def test_clamped_glu_and_embedding_into_streams(dtype):
     ops.clamped_glu(h.to(DEV), torch.cat([wg, wu]).to(DEV), out, 1.702, limit)
     want = R.clamped_glu(h.double().numpy(), wg.double().numpy(), wu.double().numpy(), np.eye(F), limit)
     close(out.float().cpu(), want, dtype, "glu")
+    if dtype == "bfloat16":       # the activation alone on gate and up rows kept in 16 bits
+        gu = torch.cat([h.float() @ wg.float().T, h.float() @ wu.float().T], dim=1).to(tdt)
+        ops.clamped_glu_mul(gu.to(DEV), out, 1.702, limit)
+        g, u = gu.double().numpy()[:, :F], gu.double().numpy()[:, F:]
+        g, u = np.minimum(g, limit), np.clip(u, -limit, limit)
+        close(out.float().cpu(), g / (1 + np.exp(-1.702 * g)) * (u + 1), dtype, "activation")
     assert float(want.max()) > 0.7 * 1.8 * 0.8 and float(np.abs(h.double().numpy() @ wg.double().numpy().T).max()) > limit
     # embedding rows, normalised, into every stream
     V, S = 19, 3
