@@ -267,11 +267,12 @@ constexpr int PROW = 64 + 8;  // bfloat16 of a row of a wave's weights in LDS
 constexpr int NW = DT / WAVE;
 
 // grid: rows x G x n_splits, 4 waves a block.  Split s of a row takes the keys at positions a0 + s * kps ..
-// a0 + (s + 1) * kps - 1 that the row sees, a0 being the row's first key rounded down to a multiple of 256 (kps is a
-// multiple of 256; pages are powers of two up to 256, so 8 consecutive positions from a multiple of 8 on lie in one
-// page); of every 256 of them wave w takes keys 64 w .. 64 w + 63.  A wave is a part of its own: it leaves, per query
-// head of the group, the maximum score m, sum exp(s - m) and sum exp(s - m) v of its keys in `parts`
-// [row][head][4 s + w][2 + dv], and no wave waits for another.
+// a0 + (s + 1) * kps - 1 that the row sees, a0 being the row's first key rounded down to a multiple of 256 and kps the
+// multiple of 256 that spreads this row's keys over the splits (pages are powers of two up to 256, so 8 consecutive positions from a multiple of 8 on lie in one
+// page); of every 256 of them wave w takes keys 64 w .. 64 w + 63.  A wave works for itself, with a running maximum
+// and sum of its own, and no wave waits for another until the end, where the block's 4 add up through LDS: the block
+// leaves, per query head of the group, the maximum score m, sum exp(s - m) and sum exp(s - m) v of its keys in
+// `parts` [row][head][split][2 + dv].
 // 64 keys: scores with all heads of the group as S = K Q^T (keys as the rows of 4 tiles, straight from the pages into
 // the operand), maxima and sums with a key a lane, weights to LDS in bfloat16, then O^T += V^T P^T over the 64 keys for
 // every 16 value elements (8 slots of an element a lane, straight from the pages).
@@ -280,7 +281,7 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     const bf16_t* __restrict__ q, int ldq, int H, int G, int dk, int dv, const bf16_t* __restrict__ cache, int P,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ positions,
     const int* __restrict__ row_seg, const int* __restrict__ rows, int mask, int mask_size, float scale, int n_splits,
-    int kps, float* __restrict__ parts) {
+    float* __restrict__ parts) {
   __shared__ __attribute__((aligned(16))) float sc_all[NW][HGMAX * SROW];
   __shared__ __attribute__((aligned(16))) bf16_t ps_all[NW][HGMAX * PROW];
   __shared__ float ml_all[NW][HGMAX][3];        // running maximum, running sum, the last pass's factor
@@ -313,6 +314,10 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
   for (int i = 0; i < ET; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
   wave_lds_order();
 
+  // the row's own keys in n_splits ranges of whole passes: a step's rows differ in length, and the launch is made for
+  // the longest the step may hold
+  const int row_passes = (pos + 1 - a0 + DT - 1) / DT;
+  const int kps = (row_passes + n_splits - 1) / n_splits * DT;
   const int lo_t = a0 + split * kps;
   const int hi_t = min(lo_t + kps, pos + 1);
   for (int t0 = lo_t + wave * WAVE; t0 < hi_t; t0 += DT) {
@@ -328,7 +333,7 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const int c = ks * 32 + lc * 8;
-          kf[tt][ks] = (seen && c < dk) ? load_frag(kp + c) : zero_frag();
+          kf[tt][ks] = (seen && c < dk) ? load_frag_once(kp + c) : zero_frag();
         }
       }
 #pragma unroll
@@ -350,7 +355,7 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
       for (int kk = 0; kk < 2; ++kk) {
         const int tp = t0 + kk * 32 + lc * 8;
         if (e < dv && tp <= pos && tp + 8 > first) {
-          vf[i][kk] = load_frag(head + (size_t)bt[tp / P] * page_stride + (size_t)P * dk + (size_t)e * P + tp % P);
+          vf[i][kk] = load_frag_once(head + (size_t)bt[tp / P] * page_stride + (size_t)P * dk + (size_t)e * P + tp % P);
           if (tp < first || tp + 8 > pos + 1) keep_positions(vf[i][kk], first - tp, pos - tp + 1);
         } else {
           vf[i][kk] = zero_frag();
@@ -387,24 +392,42 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     }
     wave_lds_order();
   }
+  // The block's 4 waves add up through LDS, 4 heads at a time, and leave one part.
   // lane: elements i * 16 + lc * 4 + 0..3 of head li
-  const int n_parts = n_splits * NW, part = split * NW + wave;
-  if (li < per) {
-    float* p = parts + (((size_t)ri * H + g * per + li) * n_parts + part) * (dv + 2);
+  constexpr int HR = 4;
+  __shared__ __attribute__((aligned(16))) float ox[NW][HR][ET * 16];
+  for (int j0 = 0; j0 < per; j0 += HR) {
+    if (li >= j0 && li < j0 + HR) {
 #pragma unroll
-    for (int i = 0; i < ET; ++i) {
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const int e = i * 16 + lc * 4 + rr;
-        if (e < dv) p[2 + e] = o[i][rr];
-      }
+      for (int i = 0; i < ET; ++i)
+        *reinterpret_cast<float4*>(&ox[wave][li - j0][i * 16 + lc * 4]) = float4{o[i][0], o[i][1], o[i][2], o[i][3]};
     }
-    if (lc == 0) { p[0] = ml[li][0]; p[1] = ml[li][1]; }
+    __syncthreads();
+    const int nh = min(HR, per - j0);
+    for (int idx = tid; idx < nh * dv; idx += DT) {
+      const int jj = idx / dv, e = idx % dv, j = j0 + jj;
+      float M = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) M = fmaxf(M, ml_all[w][j][0]);
+      float a = 0.f, l = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const float m = ml_all[w][j][0];
+        const float f = m == -INFINITY ? 0.f : __expf(m - M);
+        a = fmaf(f, ox[w][jj][e], a);
+        l = fmaf(f, ml_all[w][j][1], l);
+      }
+      float* p = parts + (((size_t)ri * H + g * per + j) * n_splits + split) * (dv + 2);
+      p[2 + e] = a;
+      if (e == 0) { p[0] = M; p[1] = l; }
+    }
+    __syncthreads();
   }
 }
 
 // out[row][head] = sum_s e^(m_s - M) o_s / (sink e^(-M) + sum_s e^(m_s - M) l_s),  M = max(m_s, 0 with a sink);
-// at most 64 parts: lane s holds part s's maximum and sum
+// at most 64 parts: lane s holds part s's maximum and sum.  The parts' elements are asked for 16 parts at a time, with
+// no condition on the way (a part beyond the last one is read as the last one, with weight 0).
 __global__ __launch_bounds__(64) void attn_masked_merge_kernel(const float* __restrict__ parts, int n_parts, int H,
                                                                int dv, const int* __restrict__ rows, int sink,
                                                                bf16_t* __restrict__ out, int ldo) {
@@ -419,14 +442,16 @@ __global__ __launch_bounds__(64) void attn_masked_merge_kernel(const float* __re
   const float L = wave_sum(w * l) + (sink ? __expf(-M) : 0.f);
   const float inv = 1.0f / L;
   for (int e0 = 0; e0 < dv; e0 += WAVE) {
-    const int e = e0 + lane;
+    const int e = min(e0 + lane, dv - 1);
     float a = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < n_parts; ++s) {
-      const float ws = __shfl(w, s, WAVE);
-      if (e < dv) a = fmaf(ws, p[(size_t)s * (dv + 2) + 2 + e], a);
+    for (int s0 = 0; s0 < n_parts; s0 += 16) {
+      float v[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) v[k] = p[(size_t)min(s0 + k, n_parts - 1) * (dv + 2) + 2 + e];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) a = fmaf(s0 + k < n_parts ? __shfl(w, (s0 + k) & 63, WAVE) : 0.f, v[k], a);
     }
-    if (e < dv) out[(size_t)r * ldo + (size_t)h * dv + e] = float_to_bf16(a * inv);
+    if (e0 + lane < dv) out[(size_t)r * ldo + (size_t)h * dv + e] = float_to_bf16(a * inv);
   }
 }
 
@@ -482,26 +507,24 @@ APC_EXPORT int apc_attention_masked_prefill_bf16(const void* q, int ldq, void* o
   return 0;
 }
 
-// `rows`: the step's rows that are decoded ones (nullptr: all n_rows rows); `keys_per_split`: a multiple of 256;
-// at most 16 splits; `parts`: room for n_rows * H * 4 * n_splits * (dv + 2) floats.
+// `rows`: the step's rows that are decoded ones (nullptr: all n_rows rows); at most 64 splits; `parts`: room for n_rows * H * n_splits * (dv + 2) floats.
 APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* out, int ldo, int n_rows, int H, int G,
                                                 int dk, int dv, const void* cache, int page_tokens,
                                                 const int* block_table, int max_blocks, const int* positions,
                                                 const int* row_seg, const int* rows, int mask, int mask_size, int sink,
-                                                float scale, int n_splits, int keys_per_split, float* parts,
-                                                hipStream_t stream) {
+                                                float scale, int n_splits, float* parts, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale);
   if (e) return e;
   if (!apc_attention_masked_takes(H, G, dk, dv, page_tokens)) return APC_ERR_UNSUPPORTED;
-  if (n_splits <= 0 || n_splits * NW > WAVE || keys_per_split <= 0 || keys_per_split % DT || !parts || max_blocks <= 0 ||
+  if (n_splits <= 0 || n_splits > WAVE || !parts || max_blocks <= 0 ||
       (long)n_rows * G * n_splits > 0x7fffffffL || H > 65535)
     return APC_ERR_BAD_ARG;
   dim3 grid(n_rows * G * n_splits), block(DT);
 #define MD_LAUNCH(KS_, ET_)                                                                                       \
   hipLaunchKernelGGL((attn_masked_decode_kernel<KS_, ET_>), grid, block, 0, stream, (const bf16_t*)q, ldq, H, G, dk, \
                      dv, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg, rows, mask,  \
-                     mask_size, scale, n_splits, keys_per_split, parts)
+                     mask_size, scale, n_splits, parts)
 #define MD_VALUES(KS_)                     \
   do {                                     \
     if (dv <= 64) MD_LAUNCH(KS_, 4);       \
@@ -514,7 +537,7 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
 #undef MD_VALUES
 #undef MD_LAUNCH
   APC_LAUNCH_CHECK();
-  hipLaunchKernelGGL(attn_masked_merge_kernel, dim3(n_rows, H), dim3(64), 0, stream, parts, n_splits * NW, H, dv, rows, sink,
+  hipLaunchKernelGGL(attn_masked_merge_kernel, dim3(n_rows, H), dim3(64), 0, stream, parts, n_splits, H, dv, rows, sink,
                      (bf16_t*)out, ldo);
   APC_LAUNCH_CHECK();
   return 0;

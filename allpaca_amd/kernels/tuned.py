@@ -456,8 +456,8 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
     return True
 
 
-MASKED_DECODE_BLOCKS = 512    # blocks the decoded rows' key ranges are cut for (2 a compute unit are resident)
-MASKED_DECODE_SPLITS = 16     # at most: a block's 4 waves are a part each, and the adding kernel takes 64 parts
+MASKED_DECODE_BLOCKS = 768    # blocks the decoded rows' key ranges are cut for (3 a compute unit are resident)
+MASKED_DECODE_SPLITS = 64     # at most: the adding kernel takes 64 parts
 
 
 def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens, block_table, step,
@@ -491,12 +491,11 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
         keys = min(step.max_decode_context, mask_size) if code else step.max_decode_context
         passes = -(-(keys + 255) // 256)        # a row's first pass starts at a multiple of 256 at or below its first key
         splits = max(1, min(passes, MASKED_DECODE_SPLITS, MASKED_DECODE_BLOCKS // max(1, n * n_kv_heads)))
-        kps = -(-passes // splits) * 256
-        parts = torch.empty(n * n_heads * 4 * splits * (value_dim + 2), dtype=torch.float32, device=q.device)
+        parts = torch.empty(n * n_heads * splits * (value_dim + 2), dtype=torch.float32, device=q.device)
         _lib.check(L.apc_attention_masked_decode_bf16(
             q.data_ptr(), ldq, out.data_ptr(), ldo, n, n_heads, n_kv_heads, key_dim, value_dim, cache.data_ptr(),
             page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
             step.row_seg.data_ptr(), step.decode_rows.data_ptr() if step.decode_rows is not None else 0, code,
-            int(mask_size), 1 if sink else 0, float(scale), splits, kps, parts.data_ptr(), stream),
+            int(mask_size), 1 if sink else 0, float(scale), splits, parts.data_ptr(), stream),
             "attention_masked_decode_bf16")
     return True
