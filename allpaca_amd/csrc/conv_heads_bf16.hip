@@ -1,5 +1,5 @@
 // The short convolution on the heads of projected rows (see plain_mixers.hip for the formulas) for bfloat16 rows, 16
-// bytes a thread: a block takes ROWS (2 or 4) consecutive rows whole, a thread PPT pieces of 8 channels of each, with the taps of
+// bytes a thread: a block takes 8 or 4 consecutive rows whole, a thread PPT pieces of 8 channels of each, with the taps of
 // its channels in registers.  Sums of squares of the pieces go through LDS, so a head may be any multiple of 8 wide.
 // The row holds q heads, then k heads, then v heads.  The state of the convolution is moved on by the plain kernel.
 #include "mfma.h"
@@ -17,8 +17,8 @@ __device__ __forceinline__ void unpack8(const Frag& f, float* v) {
   }
 }
 
-template <int PPT, int ROWS, int TAPS>
-__global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
+template <int NT, int PPT, int ROWS, int TAPS>
+__global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
     const bf16_t* __restrict__ proj, int ld, int n_rows, int H, int G, int dk, int dv, const float* __restrict__ bias,
     const float* __restrict__ conv_w, const float* __restrict__ state, int width,
     const int* __restrict__ row_seg, const int* __restrict__ seg_row0, const int* __restrict__ slots,
@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
   float y[PPT][ROWS][8];
 #pragma unroll
   for (int k = 0; k < PPT; ++k) {
-    const int p = tid + 256 * k;
+    const int p = tid + NT * k;
     if (p >= pieces) continue;
     const int c0 = p * 8;
     float b[8], w[8 * TAPS];                         // w[e * TAPS + j], as the taps lie in memory
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
   const int kq = H * dk, kk = (H + G) * dk;
 #pragma unroll
   for (int k = 0; k < PPT; ++k) {
-    const int p = tid + 256 * k;
+    const int p = tid + NT * k;
     if (p >= pieces) continue;
     const int c0 = p * 8;
     const int kind = c0 < kq ? 0 : c0 < kk ? 1 : 2;
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256) void conv_heads_bf16_kernel(
 // 1 if the kernel takes these sizes (q, k and v heads side by side from column 0 on), else 0
 APC_EXPORT int apc_conv_heads_bf16_takes(int ld, int width, int H, int G, int dk, int dv, int taps, int ldq) {
   if (H <= 0 || G < 0 || dk % 8 || (G && dv % 8) || taps < 1 || taps > MAXT || ld % 8 || ldq % 8) return 0;
-  if (width != H * dk + G * (dk + dv) || width / 8 > 8 * 256) return 0;
+  if (width != H * dk + G * (dk + dv) || width / 8 > 2 * 768) return 0;
   return 1;
 }
 
@@ -192,26 +192,39 @@ APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, 
     return APC_ERR_UNSUPPORTED;
   if (taps > 1 && (!conv_w || !state || !slots)) return APC_ERR_BAD_ARG;
   if (G > 0 && (!cache || !block_table || page_tokens <= 0 || max_blocks <= 0)) return APC_ERR_BAD_ARG;
+  // A row's pieces of 8 channels are spread over up to 768 threads (a block of 1,024 would leave a thread too few
+  // registers): a thread's pieces come one after the other, each with loads of its own to wait for.
   const int pieces = width / 8;
-  const int ppt = (pieces + 255) / 256;
-  const int rows_a_block = ppt <= 4 ? 4 : 2;   // (a thread keeps its channels' taps for all rows of the block)
-  dim3 grid((n_rows + rows_a_block - 1) / rows_a_block), block(256);
+  const int nt = pieces <= 256 ? 256 : pieces <= 512 ? 512 : pieces <= 768 ? 768 : pieces <= 1024 ? 512 : 768;
+  // (a thread keeps its channels' taps for all rows of the block: 8 rows where a thread has one piece, else 4; a step
+  // of few rows, decoded ones, has a block a row: the rows of a block come one after the other)
+  const bool few = n_rows <= 32;
+  const int rows_a_block = few ? 1 : pieces <= 768 ? 8 : 4;
+  dim3 grid((n_rows + rows_a_block - 1) / rows_a_block), block(nt);
   const size_t lds = (size_t)rows_a_block * pieces * sizeof(float);
-#define CH_LAUNCH(PPT_, ROWS_, TAPS_)                                                                              \
-  hipLaunchKernelGGL((conv_heads_bf16_kernel<PPT_, ROWS_, TAPS_>), grid, block, lds, stream, (const bf16_t*)proj,  \
-                     ld, n_rows, H, G, dk, dv, bias, conv_w, state, width, row_seg, seg_row0, slots, positions,     \
-                     unit_norm, eps, (bf16_t*)q_out, ldq, block_table, max_blocks, (bf16_t*)cache, page_tokens)
-#define CH_TAPS(PPT_, ROWS_)                            \
-  do {                                                  \
-    if (taps == 1) CH_LAUNCH(PPT_, ROWS_, 1);           \
-    else if (taps == 2) CH_LAUNCH(PPT_, ROWS_, 2);      \
-    else if (taps == 3) CH_LAUNCH(PPT_, ROWS_, 3);      \
-    else CH_LAUNCH(PPT_, ROWS_, 4);                     \
+#define CH_LAUNCH(NT_, PPT_, ROWS_, TAPS_)                                                                          \
+  hipLaunchKernelGGL((conv_heads_bf16_kernel<NT_, PPT_, ROWS_, TAPS_>), grid, block, lds, stream,                   \
+                     (const bf16_t*)proj, ld, n_rows, H, G, dk, dv, bias, conv_w, state, width, row_seg, seg_row0,  \
+                     slots, positions, unit_norm, eps, (bf16_t*)q_out, ldq, block_table, max_blocks, (bf16_t*)cache, \
+                     page_tokens)
+#define CH_TAPS(NT_, PPT_, ROWS_)                            \
+  do {                                                       \
+    if (taps == 1) CH_LAUNCH(NT_, PPT_, ROWS_, 1);           \
+    else if (taps == 2) CH_LAUNCH(NT_, PPT_, ROWS_, 2);      \
+    else if (taps == 3) CH_LAUNCH(NT_, PPT_, ROWS_, 3);      \
+    else CH_LAUNCH(NT_, PPT_, ROWS_, 4);                     \
   } while (0)
-  if (ppt <= 1) CH_TAPS(1, 4);
-  else if (ppt <= 2) CH_TAPS(2, 4);
-  else if (ppt <= 4) CH_TAPS(4, 4);
-  else CH_TAPS(8, 2);
+#define CH_ROWS(NT_, PPT_, ROWS_)            \
+  do {                                       \
+    if (few) CH_TAPS(NT_, PPT_, 1);          \
+    else CH_TAPS(NT_, PPT_, ROWS_);          \
+  } while (0)
+  if (pieces <= 256) CH_ROWS(256, 1, 8);
+  else if (pieces <= 512) CH_ROWS(512, 1, 8);
+  else if (pieces <= 768) CH_ROWS(768, 1, 8);
+  else if (pieces <= 1024) CH_ROWS(512, 2, 4);
+  else CH_ROWS(768, 2, 4);
+#undef CH_ROWS
 #undef CH_TAPS
 #undef CH_LAUNCH
   APC_LAUNCH_CHECK();

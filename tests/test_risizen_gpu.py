@@ -37,7 +37,9 @@ def make_step(segments, page_tokens, tables, slots):
 
 
 # =========================================================================================== kernels alone
-@pytest.mark.parametrize("taps, H, G, dk, dv", [(4, 3, 1, 24, 16), (2, 2, 2, 8, 40), (1, 2, 1, 16, 16), (3, 2, 0, 72, 0)])
+@pytest.mark.parametrize("taps, H, G, dk, dv", [(4, 3, 1, 24, 16), (2, 2, 2, 8, 40), (1, 2, 1, 16, 16), (3, 2, 0, 72, 0),
+                                                 # rows wide enough for the larger blocks of the 16-byte kernel
+                                                 (4, 32, 8, 128, 128), (3, 16, 4, 128, 64), (2, 40, 8, 128, 128)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_conv_heads_against_the_plain_convolution_and_norm(taps, H, G, dk, dv, dtype):
     """Three requests in one step: one starting (zeros ahead of it), two going on from states that an earlier step
