@@ -358,3 +358,68 @@ def test_greedy_generation_through_the_engine():
             outs = engine.generate(prompts, GenerationParams(max_tokens=12, temperature=0.0))
             for p, o in zip(prompts, outs):
                 assert o.token_ids == R.greedy(cfg, w, p, 12), (name, graphs, len(p))
+
+
+def test_command_line_generates_with_the_design():
+    """The command line on a model folder of the design (float32, greedy: the plain implementation's tokens) and on
+    the design's preset with random weights."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = model_folder("RA")
+    cfg, w = oracle(folder)
+    prompts = [tokens_for("RA", 7, 5), tokens_for("RA", 19, 6)]
+    spec = ";".join(",".join(str(t) for t in p) for p in prompts)
+    cmd = [sys.executable, os.path.join(root, "bin", "allpaca-amd"), "generate", "--model", folder, "--dtype", "fp32",
+           "--prompt-tokens", spec, "--max-tokens", "6", "--temperature", "0", "--json"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    outs = [json.loads(ln) for ln in r.stdout.strip().splitlines() if ln.startswith("{")]
+    assert [o["token_ids"] for o in outs] == [R.greedy(cfg, w, p, 6) for p in prompts]
+    cmd = [sys.executable, os.path.join(root, "bin", "allpaca-amd"), "generate", "--synthetic", "risizen-tiny",
+           "--prompt-tokens", "1,2,3;4,5", "--max-tokens", "5", "--temperature", "0", "--json"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    outs = [json.loads(ln) for ln in r.stdout.strip().splitlines() if ln.startswith("{")]
+    assert len(outs) == 2 and all(len(o["token_ids"]) == 5 for o in outs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_tool_with_two_slots_and_a_small_pool(tmp_path, dtype):
+    """The replay program on a model folder of the design: three requests through two state slots and a pool that holds
+    two of them, portions beside single tokens, a request left out of a step; its files against the plain logits."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    name = "RC"
+    folder = model_folder(name)
+    a, b, c = tokens_for(name, 70, 31), tokens_for(name, 9, 32), tokens_for(name, 50, 33)
+    steps = [
+        dict(step=0, entries=[dict(id="a", tokens=a[:33], want=list(range(33))), dict(id="b", tokens=b[:1], want=[0])], end=[]),
+        dict(step=1, entries=[dict(id="b", tokens=b[1:3], want=[0, 1])], end=[]),
+        dict(step=2, entries=[dict(id="a", tokens=a[33:69], want=list(range(36))), dict(id="b", tokens=b[3:], want=list(range(6)))],
+             end=["b"]),
+        dict(step=3, entries=[dict(id="a", tokens=a[69:], want=[0]), dict(id="c", tokens=c[:2], want=[0, 1])], end=["a"]),
+        dict(step=4, entries=[dict(id="c", tokens=c[2:], want=list(range(48)))], end=["c"]),
+    ]
+    out = str(tmp_path / "replay")
+    cmd = [sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", out,
+           "--max-tokens", "192", "--max-live", "2", "--poison-free-pages"]
+    r = subprocess.run(cmd, input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=280)
+    assert r.returncode == 0, r.stderr[-3000:]
+    assert [ln for ln in r.stdout.split("\n") if ln.startswith("done")] == [f"done {i}" for i in range(5)]
+    V = CONFIGS[name][0]["vocab"]
+    got = {k: [] for k in "abc"}
+    for s in steps:
+        rows = np.fromfile(os.path.join(out, f"{s['step']}.f32"), dtype="<f4").reshape(-1, V)
+        at = 0
+        for e in s["entries"]:
+            got[e["id"]].append(rows[at:at + len(e["want"])])
+            at += len(e["want"])
+        assert at == rows.shape[0]
+    for k, toks in zip("abc", (a, b, c)):
+        close(np.concatenate(got[k]), oracle_logits(folder, toks), dtype, f"replay {k}")
