@@ -54,12 +54,15 @@ __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
       const float4 a = *reinterpret_cast<const float4*>(bias + c0), c = *reinterpret_cast<const float4*>(bias + c0 + 4);
       b[0] = a.x; b[1] = a.y; b[2] = a.z; b[3] = a.w; b[4] = c.x; b[5] = c.y; b[6] = c.z; b[7] = c.w;
     }
-    if (TAPS > 1) {
+    if (conv_w) {
 #pragma unroll
       for (int i = 0; i < 2 * TAPS; ++i) {
         const float4 a = *reinterpret_cast<const float4*>(conv_w + (size_t)c0 * TAPS + 4 * i);
         w[4 * i] = a.x; w[4 * i + 1] = a.y; w[4 * i + 2] = a.z; w[4 * i + 3] = a.w;
       }
+    } else {                                         // no convolution (one tap of 1)
+#pragma unroll
+      for (int i = 0; i < 8 * TAPS; ++i) w[i] = 1.f;
     }
     // The rows' inputs are asked for together and used afterwards, so the loads are in flight at once.  When every row
     // of the block has its TAPS - 1 predecessors in its own segment (all but the first rows of a prompt portion), the
@@ -79,7 +82,7 @@ __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
           float u[8];
           unpack8(src[rr + j], u);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) acc[e] = TAPS > 1 ? fmaf(w[e * TAPS + j], u[e] + b[e], acc[e]) : u[e] + b[e];
+          for (int e = 0; e < 8; ++e) acc[e] = fmaf(w[e * TAPS + j], u[e] + b[e], acc[e]);
         }
         float ss = 0.f;
 #pragma unroll
@@ -119,7 +122,7 @@ __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
             u[4] = sb[j].x; u[5] = sb[j].y; u[6] = sb[j].z; u[7] = sb[j].w;
           }
 #pragma unroll
-          for (int e = 0; e < 8; ++e) acc[e] = TAPS > 1 ? fmaf(w[e * TAPS + j], u[e], acc[e]) : u[e];
+          for (int e = 0; e < 8; ++e) acc[e] = fmaf(w[e * TAPS + j], u[e], acc[e]);
         }
         float ss = 0.f;
 #pragma unroll
@@ -191,6 +194,7 @@ APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, 
       ((uintptr_t)bias & 15u) || ((uintptr_t)conv_w & 15u))
     return APC_ERR_UNSUPPORTED;
   if (taps > 1 && (!conv_w || !state || !slots)) return APC_ERR_BAD_ARG;
+  if (!conv_w && taps != 1) return APC_ERR_BAD_ARG;
   if (G > 0 && (!cache || !block_table || page_tokens <= 0 || max_blocks <= 0)) return APC_ERR_BAD_ARG;
   // A row's pieces of 8 channels are spread over up to 768 threads (a block of 1,024 would leave a thread too few
   // registers): a thread's pieces come one after the other, each with loads of its own to wait for.

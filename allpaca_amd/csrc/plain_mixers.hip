@@ -8,7 +8,7 @@
 
 constexpr int MAX_TAPS = 8;
 constexpr int MAX_PER_LANE = 4;   // head sizes up to 256
-constexpr int MAX_STREAMS = 8;
+constexpr int MAX_STREAMS = 16;
 
 // ---------------------------------------------------------------------------
 // Short convolution on the heads of a projected row, then (q, k) unit RMS norm per head, then q to `q_out` and k, v
@@ -17,7 +17,7 @@ constexpr int MAX_STREAMS = 8;
 // proj [T, ld]: q heads at column q_off (H of dk), k heads at k_off (G of dk), v heads at v_off (G of dv); with
 // G == 0 the row holds q only.  Channel c of the convolution is column c of the row:
 //   u[t][c] = proj[t][c] + bias[c]
-//   y[t][c] = sum_j w[c][j] * u[t - (n-1) + j][c]            (n taps; without w: y = u)
+//   y[t][c] = sum_j w[c][j] * u[t - (n-1) + j][c]            (n taps, n = 1 too; without w: y = u)
 // u of the n-1 positions ahead of a segment's first row comes from state[slot][n-1][width] (zero for a new request:
 // the sequence starts with zeros).  `conv_state_kernel` moves the state on afterwards.
 //   q, k:  y / sqrt(mean_head(y^2) + eps)  if `unit_norm`
@@ -49,7 +49,7 @@ __global__ __launch_bounds__(64) void conv_heads_kernel(
       const int c = col0 + i;
       const float b = bias ? bias[c] : 0.f;
       float acc;
-      if (taps > 1) {
+      if (conv_w) {
         acc = 0.f;
         for (int j = 0; j < taps; ++j) {          // oldest first: the order of the sum is that of the taps
           const int back = taps - 1 - j;

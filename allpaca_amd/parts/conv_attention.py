@@ -2,7 +2,8 @@
 
 Per row, with h the mixer's input:
   u_q = Wq h + bq, u_k = Wk h + bk, u_v = Wv h + bv                       (biases optional)
-  c_x[t] = sum_j conv_x[:, j] * u_x[t - (taps - 1) + j]                   (zeros ahead of the sequence; taps 0: c = u)
+  c_x[t] = sum_j conv_x[:, j] * u_x[t - (taps - 1) + j]                   (zeros ahead of the sequence; taps 0: c = u,
+                                                                            no tensor; 1 tap is a scale per channel)
   q, k = c_q, c_k divided by their root mean square over a head           (`unit_norm`)
   s = (q . k) * scale over the keys that the mask lets the row see: all earlier ones ("causal"), the last n
       ("window") or those of the row's own chunk of n positions counted from position 0 ("chunk")
@@ -56,7 +57,7 @@ class ConvAttention(Mixer):
             out[n[p]] = ParamSpec((rows, self.D))
             if self.bias:
                 out[n[p] + n["bias"]] = ParamSpec((rows,), store="float32", init="zeros")
-            if self.taps > 1:
+            if self.taps >= 1:
                 out[n[p] + n["conv"]] = ParamSpec((rows, self.taps), store="float32", init="normal")
         out[n["o"]] = ParamSpec((self.D, self.H * self.dv))
         return out
@@ -79,7 +80,7 @@ class ConvAttention(Mixer):
         if self.bias:
             self.b_in = torch.cat([to_device(tensors[n[p] + n["bias"]], rt, torch.float32)
                                    for p, _ in self.projections]).contiguous()
-        if self.taps > 1:
+        if self.taps >= 1:
             self.conv_w = torch.cat([to_device(tensors[n[p] + n["conv"]], rt, torch.float32)
                                      for p, _ in self.projections], dim=0).contiguous()
 

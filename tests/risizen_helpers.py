@@ -49,10 +49,10 @@ TINY_RC = dict(
     layers=[_layer(_att(4, 2, 64, 32, 0.15, conv=4, chunk=48), ff=256, limit=1.5),
             _layer(_att(8, 2, 32, 64, 0.2, conv=4, chunk=80), ff=192, limit=1.5),
             _layer(_att(8, 2, 32, 64, 0.2, conv=4, chunk=80, kv_from=1), ff=192, limit=1.5)])
-# D: no `streams` key at all (the plain residual sum, no connection tensors), no mask, a layer without convolution
+# D: no `streams` key at all (the plain residual sum, no connection tensors), no mask, a convolution of a single tap
 TINY_RD = dict(
     architecture="Risizen", vocab=50, width=32, norm=dict(eps=1e-6), logit_scale=2.0,
-    layers=[_layer(_att(2, 2, 16, 16, 0.3), ff=48, limit=1.0), _layer(_att(2, 1, 16, 8, 0.3, conv=2, kv_from=None))])
+    layers=[_layer(_att(2, 2, 16, 16, 0.3, conv=1), ff=48, limit=1.0), _layer(_att(2, 1, 16, 8, 0.3, conv=2, kv_from=None))])
 
 CONFIGS = {"RA": (TINY_RA, 11), "RB": (TINY_RB, 12), "RC": (TINY_RC, 13), "RD": (TINY_RD, 14)}
 

@@ -37,7 +37,7 @@ def make_step(segments, page_tokens, tables, slots):
 
 
 # =========================================================================================== kernels alone
-@pytest.mark.parametrize("taps, H, G, dk, dv", [(4, 3, 1, 24, 16), (2, 2, 2, 8, 40), (1, 2, 1, 16, 16), (3, 2, 0, 72, 0),
+@pytest.mark.parametrize("taps, H, G, dk, dv", [(4, 3, 1, 24, 16), (2, 2, 2, 8, 40), (1, 2, 1, 16, 16), (0, 2, 1, 16, 24), (3, 2, 0, 72, 0),
                                                  # rows wide enough for the larger blocks of the 16-byte kernel
                                                  (4, 32, 8, 128, 128), (3, 16, 4, 128, 64), (2, 40, 8, 128, 128)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -56,13 +56,14 @@ def test_conv_heads_against_the_plain_convolution_and_norm(taps, H, G, dk, dv, d
     tdt = DTYPES[dtype]
     proj = torch.as_tensor(rng.normal(size=(T, width)), dtype=torch.float32).to(tdt)
     bias = rng.normal(size=width).astype(np.float32)
-    conv = rng.normal(size=(width, taps)).astype(np.float32) if taps > 1 else None
+    conv = rng.normal(size=(width, taps)).astype(np.float32) if taps >= 1 else None     # 0: no convolution at all
+    taps = max(taps, 1)
     state0 = rng.normal(size=(4, max(taps - 1, 1), width)).astype(np.float32)
     state0[2] = 0.0                                             # the slot of the request that starts
     state = dev(state0[:, :taps - 1]) if taps > 1 else None
     q_out = torch.empty((T, H * dk), dtype=tdt, device=DEV)
     cache = torch.zeros((8, max(G, 1), P_ * (dk + dv)), dtype=tdt, device=DEV) if G else None
-    ops.conv_heads(proj.to(DEV), 0, H * dk, (H + G) * dk, H, G, dk, dv, dev(bias), dev(conv) if taps > 1 else None,
+    ops.conv_heads(proj.to(DEV), 0, H * dk, (H + G) * dk, H, G, dk, dv, dev(bias), dev(conv) if conv is not None else None,
                    state, step, step.state_slots, True, eps, q_out, step.block_tables[0] if G else None, cache, P_)
     torch.cuda.synchronize()
     u_all = proj.float().numpy().astype(np.float64) + bias
@@ -70,7 +71,7 @@ def test_conv_heads_against_the_plain_convolution_and_norm(taps, H, G, dk, dv, d
     for (pos0, n), slot, table in zip(segs, slots, tables):
         u = u_all[r0:r0 + n]
         before = state0[slot, :taps - 1].astype(np.float64)
-        y = R.short_conv(u, conv.astype(np.float64), before) if taps > 1 else u
+        y = R.short_conv(u, conv.astype(np.float64), before) if conv is not None else u
         close(q_out[r0:r0 + n].float().cpu(), R.unit_rms(y[:, :H * dk].reshape(n, H, dk), eps).reshape(n, -1), dtype, "q")
         if taps > 1:
             want_state = np.concatenate([before, u])[-(taps - 1):]
@@ -176,7 +177,7 @@ def test_one_key_stands_out(mask, size, pos, key, seen, rows, dtype):
     assert hit == seen, (last[0, :3], seen)
 
 
-@pytest.mark.parametrize("S, D", [(1, 40), (2, 192), (3, 1000), (4, 64), (2, 50), (3, 4100), (8, 8192)])
+@pytest.mark.parametrize("S, D", [(1, 40), (2, 192), (3, 1000), (4, 64), (2, 50), (3, 4100), (8, 8192), (12, 64), (16, 30)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_streams_read_write_and_both(S, D, dtype):
     from allpaca_amd.kernels import ops

@@ -12,6 +12,7 @@ from risizen_helpers import CONFIGS, TINY_RA, TINY_RB, TINY_RD, model_folder, or
 
 from allpaca_amd.config import ConfigError
 from allpaca_amd.models import DecoderModel, describe_model
+from allpaca_amd.parts import PagedKeysValues
 
 
 # ------------------------------------------------------------------------------------------- the plain mechanisms
@@ -95,7 +96,9 @@ def test_config_is_read_whole():
     assert cfg.layers[3].mlp.limit == 0.5 and cfg.layers[0].mlp.ff == 80
     assert [e.cache_of for e in spec.plan] == [None, 0, None, 2] and spec.streams == 3
     _, cfg, spec = describe_model(TINY_RD)
-    assert cfg.streams == 1 and not cfg.has_stream_weights and cfg.layers[0].mixer.conv == 0
+    assert cfg.streams == 1 and not cfg.has_stream_weights and cfg.layers[0].mixer.conv == 1
+    ps = DecoderModel(spec).param_specs()
+    assert ps["l0.mix.q.conv"].shape == (32, 1) and DecoderModel(spec).cache_needs()[0] == PagedKeysValues(2, 16, 16)
 
 
 @pytest.mark.parametrize("change, word", [
