@@ -1,7 +1,8 @@
 // The short convolution on the heads of projected rows (see plain_mixers.hip for the formulas) for bfloat16 rows, 16
 // bytes a thread: a block takes 8 or 4 consecutive rows whole, a thread PPT pieces of 8 channels of each, with the taps of
 // its channels in registers.  Sums of squares of the pieces go through LDS, so a head may be any multiple of 8 wide.
-// The row holds q heads, then k heads, then v heads.  The state of the convolution is moved on by the plain kernel.
+// The row holds q heads, then k heads, then v heads.  The state of the convolution is moved on by the plain kernel,
+// or here (`fold_state`) in a step of few rows in which every segment is a single row (decoded tokens).
 #include "mfma.h"
 #include <math.h>
 
@@ -20,7 +21,7 @@ __device__ __forceinline__ void unpack8(const Frag& f, float* v) {
 template <int NT, int PPT, int ROWS, int TAPS>
 __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
     const bf16_t* __restrict__ proj, int ld, int n_rows, int H, int G, int dk, int dv, const float* __restrict__ bias,
-    const float* __restrict__ conv_w, const float* __restrict__ state, int width,
+    const float* __restrict__ conv_w, float* __restrict__ state, int fold_state, int width,
     const int* __restrict__ row_seg, const int* __restrict__ seg_row0, const int* __restrict__ slots,
     const int* __restrict__ positions, int unit_norm, float eps, bf16_t* __restrict__ q_out, int ldq,
     const int* __restrict__ block_table, int max_blocks, bf16_t* __restrict__ cache, int P) {
@@ -123,6 +124,14 @@ __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
           }
 #pragma unroll
           for (int e = 0; e < 8; ++e) acc[e] = fmaf(w[e * TAPS + j], u[e], acc[e]);
+          // A step in which every segment is one row: the row's state moves on here (this thread alone reads and
+          // writes these channels of the row's slot, and it has read them all): rows 1 .. of the old state become
+          // rows 0 .., the row's own input the last.
+          if (TAPS > 1 && fold_state && r0 + rr < n_rows && j >= 1) {
+            float* sp = state + ((size_t)slots[seg[rr]] * (TAPS - 1) + (j - 1)) * width + c0;
+            *reinterpret_cast<float4*>(sp) = float4{u[0], u[1], u[2], u[3]};
+            *reinterpret_cast<float4*>(sp + 4) = float4{u[4], u[5], u[6], u[7]};
+          }
         }
         float ss = 0.f;
 #pragma unroll
@@ -184,7 +193,7 @@ APC_EXPORT int apc_conv_heads_bf16_takes(int ld, int width, int H, int G, int dk
 }
 
 APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, int G, int dk, int dv, const float* bias,
-                                   const float* conv_w, int taps, const float* state, int width, const int* row_seg,
+                                   const float* conv_w, int taps, float* state, int fold_state, int width, const int* row_seg,
                                    const int* seg_row0, const int* slots, const int* positions, int unit_norm, float eps,
                                    void* q_out, int ldq, const int* block_table, int max_blocks, void* cache,
                                    int page_tokens, hipStream_t stream) {
@@ -202,13 +211,13 @@ APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, 
   const int nt = pieces <= 256 ? 256 : pieces <= 512 ? 512 : pieces <= 768 ? 768 : pieces <= 1024 ? 512 : 768;
   // (a thread keeps its channels' taps for all rows of the block: 8 rows where a thread has one piece, else 4; a step
   // of few rows, decoded ones, has a block a row: the rows of a block come one after the other)
-  const bool few = n_rows <= 32;
+  const bool few = n_rows <= 32 || fold_state;
   const int rows_a_block = few ? 1 : pieces <= 768 ? 8 : 4;
   dim3 grid((n_rows + rows_a_block - 1) / rows_a_block), block(nt);
   const size_t lds = (size_t)rows_a_block * pieces * sizeof(float);
 #define CH_LAUNCH(NT_, PPT_, ROWS_, TAPS_)                                                                          \
   hipLaunchKernelGGL((conv_heads_bf16_kernel<NT_, PPT_, ROWS_, TAPS_>), grid, block, lds, stream,                   \
-                     (const bf16_t*)proj, ld, n_rows, H, G, dk, dv, bias, conv_w, state, width, row_seg, seg_row0,  \
+                     (const bf16_t*)proj, ld, n_rows, H, G, dk, dv, bias, conv_w, state, fold_state, width, row_seg, seg_row0,  \
                      slots, positions, unit_norm, eps, (bf16_t*)q_out, ldq, block_table, max_blocks, (bf16_t*)cache, \
                      page_tokens)
 #define CH_TAPS(NT_, PPT_, ROWS_)                            \

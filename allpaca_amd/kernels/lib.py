@@ -67,7 +67,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, F, I, I, P, P],
         "apc_attention_decode_bf16": [P, I, I, P, I, I, I, I, I, P, I, P, I, P, P, P, I, F, I, I, P, P, P],
         "apc_conv_heads_bf16_takes": [I, I, I, I, I, I, I, I],
-        "apc_conv_heads_bf16": [P, I, I, I, I, I, I, P, P, I, P, I, P, P, P, P, I, F, P, I, P, I, P, I, P],
+        "apc_conv_heads_bf16": [P, I, I, I, I, I, I, P, P, I, P, I, I, P, P, P, P, I, F, P, I, P, I, P, I, P],
         "apc_attention_masked_takes": [I, I, I, I, I],
         "apc_attention_masked_prefill_bf16": [P, I, P, I, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, F, P],
         "apc_attention_masked_decode_bf16": [P, I, P, I, I, I, I, I, I, P, I, P, I, P, P, P, I, I, I, F, I, P, P],

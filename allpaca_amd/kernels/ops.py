@@ -415,16 +415,18 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
                 and proj.data_ptr() % 16 == 0 and q_out.data_ptr() % 16 == 0
                 and (cache is None or cache.data_ptr() % 16 == 0) and (state is None or state.data_ptr() % 16 == 0)
                 and (conv_w is None or (conv_w.data_ptr() % 16 == 0 and width % 4 == 0))):
-            # the same on 16 bytes a thread (library `tuned`); the plain kernel then moves the state on
+            # the same on 16 bytes a thread (library `tuned`); the plain kernel then moves the state on, unless every
+            # segment is a single row (decoded tokens): then the kernel does that too
+            fold = taps > 1 and bool(getattr(step, "decode_only", False))
             _lib.check(LT.apc_conv_heads_bf16(
                 proj.data_ptr(), ld, T, n_heads, G, key_dim, value_dim, _f32(bias, width, "bias"),
                 _f32(conv_w, width * taps, "conv weights"), taps,
-                state.data_ptr() if taps > 1 else 0, width, _i32(step.row_seg, T, "row_seg"),
+                state.data_ptr() if taps > 1 else 0, 1 if fold else 0, width, _i32(step.row_seg, T, "row_seg"),
                 _i32(step.seg_row0, S, "seg_row0"), _i32(slots, S, "slots") if taps > 1 else 0,
                 _i32(step.positions, T, "positions"), 1 if unit_norm else 0, float(eps), q_out.data_ptr(), ldq,
                 block_table.data_ptr() if G else 0, max_blocks, cache.data_ptr() if G else 0, page_tokens, _stream()),
                 "conv_heads_bf16")
-            if taps > 1:
+            if taps > 1 and not fold:
                 _lib.check(L.apc_conv_state(proj.data_ptr(), _code(proj), ld, _f32(bias, width, "bias"), taps,
                                             state.data_ptr(), width, S, _i32(step.seg_row0, S, "seg_row0"),
                                             _i32(step.seg_rows, S, "seg_rows"), _i32(slots, S, "slots"), _stream()),
