@@ -533,7 +533,7 @@ def design_point(cfg_json, dtype, batch, context, steps, warmup, T):
 
 def design_rooflines(size, layers, streams, batch, context, T, points):
     """For the kernels the new design adds and their like kernels of the llama decoder: the bytes or the arithmetic
-    of the launches of a step, over the measured time, as a share of the card's peak (8 TB/s, 2.5 PFLOP/s)."""
+    of the launches of a step, over the measured time, as a share of the GPU's peak (8 TB/s, 2.5 PFLOP/s)."""
     D, H, G, d, F, V = DESIGN_SIZES[size]
     qkv = (H + 2 * G) * d
 

@@ -146,8 +146,8 @@ def test_masked_attention_against_the_plain_one(mask, size, sink, dtype):
 
 
 @pytest.mark.parametrize("mask, size, pos, key, seen", [
-    ("chunk", 96, 95, 0, True), ("chunk", 96, 96, 95, False), ("chunk", 96, 96, 96, True), ("chunk", 96, 191, 96, True),
-    ("chunk", 96, 192, 191, False), ("chunk", 500, 499, 3, True), ("window", 33, 400, 368, True),
+    ("chunk", 80, 79, 0, True), ("chunk", 80, 80, 79, False), ("chunk", 80, 80, 80, True), ("chunk", 80, 159, 80, True),
+    ("chunk", 80, 160, 159, False), ("chunk", 500, 499, 3, True), ("window", 33, 400, 368, True),
     ("window", 33, 400, 367, False), ("causal", 0, 900, 0, True), ("causal", 0, 900, 15, True),
     ("causal", 0, 900, 16, True)])
 @pytest.mark.parametrize("rows", [1, 70])
