@@ -20,7 +20,8 @@ constexpr int MAX_STREAMS = 16;
 //   y[t][c] = sum_j w[c][j] * u[t - (n-1) + j][c]            (n taps, n = 1 too; without w: y = u)
 // u of the n-1 positions ahead of a segment's first row comes from state[slot][n-1][width] (zero for a new request:
 // the sequence starts with zeros).  `conv_state_kernel` moves the state on afterwards.
-//   q, k:  y / sqrt(mean_head(y^2) + eps)  if `unit_norm`
+//   q, k:  y / sqrt(mean(y^2) + eps)  if `unit_norm`, the mean over the head, or over each piece of `norm_dim`
+//          elements of it (norm_dim divides dk; 0: the whole head); times q_norm_w / k_norm_w [norm_dim] if given
 // pages: page = block_table[seg][pos / P]; keys page[g][slot * dk + i], values page[g][P * dk + e * P + slot]
 // (a key's elements lie together, a value element's slots lie together), a page being G * P * (dk + dv) elements.
 // ---------------------------------------------------------------------------
@@ -28,7 +29,8 @@ __global__ __launch_bounds__(64) void conv_heads_kernel(
     const void* __restrict__ proj, int in_dtype, int ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv,
     const float* __restrict__ bias, const float* __restrict__ conv_w, int taps, const float* __restrict__ state,
     int width, const int* __restrict__ row_seg, const int* __restrict__ seg_row0, const int* __restrict__ slots,
-    const int* __restrict__ positions, int unit_norm, float eps, void* __restrict__ q_out, int q_dtype, int ldq,
+    const int* __restrict__ positions, int unit_norm, float eps, int norm_dim, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, void* __restrict__ q_out, int q_dtype, int ldq,
     const int* __restrict__ block_table, int max_blocks, void* __restrict__ cache, int cache_dtype, int P) {
   const int r = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
   int kind, head, d, col0;
@@ -64,8 +66,44 @@ __global__ __launch_bounds__(64) void conv_heads_kernel(
       ss = fmaf(acc, acc, ss);
     }
   }
-  float inv = 1.f;
-  if (unit_norm && kind != 2) inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
+  if (unit_norm && kind != 2) {
+    const int nd = norm_dim > 0 ? norm_dim : d;
+    const float* nw = kind == 0 ? q_norm_w : k_norm_w;
+    if (nd == d) {
+      const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
+#pragma unroll
+      for (int e = 0; e < MAX_PER_LANE; ++e) {
+        const int i = lane + e * WAVE;
+        y[e] = y[e] * inv;
+        if (nw && i < d) y[e] *= nw[i];
+      }
+    } else {
+      float inv_mine[MAX_PER_LANE];
+#pragma unroll
+      for (int e = 0; e < MAX_PER_LANE; ++e) inv_mine[e] = 1.f;
+      for (int piece = 0; piece < d / nd; ++piece) {
+        float part = 0.f;
+#pragma unroll
+        for (int e = 0; e < MAX_PER_LANE; ++e) {
+          const int i = lane + e * WAVE;
+          if (i < d && i / nd == piece) part = fmaf(y[e], y[e], part);
+        }
+        const float inv = 1.0f / sqrtf(wave_sum(part) / (float)nd + eps);
+#pragma unroll
+        for (int e = 0; e < MAX_PER_LANE; ++e) {
+          const int i = lane + e * WAVE;
+          if (i < d && i / nd == piece) inv_mine[e] = inv;
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < MAX_PER_LANE; ++e) {
+        const int i = lane + e * WAVE;
+        y[e] = y[e] * inv_mine[e];
+        if (nw && i < d) y[e] *= nw[i % nd];
+      }
+    }
+  }
+  const float inv = 1.f;
 
   if (kind == 0) {
 #pragma unroll
@@ -117,9 +155,11 @@ APC_EXPORT int apc_conv_heads(const void* proj, int in_dtype, int ld, int q_off,
                               int n_segs, int H, int G, int dk, int dv, const float* bias, const float* conv_w,
                               int taps, float* state, int width, const int* row_seg, const int* seg_row0,
                               const int* seg_rows, const int* slots, const int* positions, int unit_norm, float eps,
+                              int norm_dim, const float* q_norm_w, const float* k_norm_w,
                               void* q_out, int q_dtype, int ldq, const int* block_table, int max_blocks, void* cache,
                               int cache_dtype, int page_tokens, hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if (norm_dim < 0 || (norm_dim > 0 && dk % norm_dim)) return APC_ERR_BAD_ARG;
   if (H <= 0 || G < 0 || dk <= 0 || (G > 0 && dv <= 0) || taps < 1 || width <= 0 || n_segs <= 0) return APC_ERR_BAD_ARG;
   if (taps > 1 && (!conv_w || !state)) return APC_ERR_BAD_ARG;
   if (G > 0 && (!cache || !block_table || page_tokens <= 0 || max_blocks <= 0)) return APC_ERR_BAD_ARG;
@@ -127,7 +167,7 @@ APC_EXPORT int apc_conv_heads(const void* proj, int in_dtype, int ld, int q_off,
     return APC_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(conv_heads_kernel, dim3(n_rows, H + 2 * G), dim3(64), 0, stream, proj, in_dtype, ld, q_off,
                      k_off, v_off, H, G, dk, dv, bias, conv_w, taps, state, width, row_seg, seg_row0, slots, positions,
-                     unit_norm, eps, q_out, q_dtype, ldq, block_table, max_blocks, cache, cache_dtype, page_tokens);
+                     unit_norm, eps, norm_dim, q_norm_w, k_norm_w, q_out, q_dtype, ldq, block_table, max_blocks, cache, cache_dtype, page_tokens);
   APC_LAUNCH_CHECK();
   if (taps > 1) {
     hipLaunchKernelGGL(conv_state_kernel, dim3(ceil_div(width, 256), n_segs), dim3(256), 0, stream, proj, in_dtype,
@@ -156,6 +196,9 @@ APC_EXPORT int apc_conv_state(const void* proj, int in_dtype, int ld, const floa
 //     mask 0: first = 0;  mask 1 (window of n): first = max(0, pos - n + 1);  mask 2 (chunks of n): first = pos - pos % n
 //   s_t = (q . K[t]) * scale;  p_t = exp(s_t) / (sink + sum exp(s_t)),  sink = 1 (a key of score 0 without a value) or 0
 //   out = sum p_t V[t];  query head h reads key/value head h / (H / G).
+// With `key_parts` = M > 1 a key of dk elements is M keys of dk / M side by side, one for each of M maps over the same
+// values: q holds H heads of dk / M elements, head j computes its scores with part j % M of the keys of kv head
+// j / (H / G) (the M heads of a group of M are the maps of one head), and `out` holds H heads of dv.
 // The running maximum starts at 0 and the running sum at 1 with a sink (the sink is the first "key"), at -inf and 0
 // without.
 // ---------------------------------------------------------------------------
@@ -163,7 +206,7 @@ __global__ __launch_bounds__(64) void masked_attention_plain_kernel(
     const void* __restrict__ q, int q_dtype, int ldq, void* __restrict__ out, int out_dtype, int ldo, int H, int G,
     int dk, int dv, const void* __restrict__ cache, int cache_dtype, int P, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ positions, const int* __restrict__ row_seg, int mask, int mask_size,
-    int sink, float scale) {
+    int sink, float scale, int key_parts) {
   __shared__ float qs[MAX_PER_LANE * WAVE];
   __shared__ float ps[WAVE];
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -176,7 +219,8 @@ __global__ __launch_bounds__(64) void masked_attention_plain_kernel(
   const size_t page_elems = (size_t)G * P * (dk + dv);
   const size_t head_off = (size_t)g * P * (dk + dv);
 
-  for (int i = lane; i < dk; i += WAVE) qs[i] = load_f(q, q_dtype, (size_t)r * ldq + (size_t)h * dk + i);
+  const int dq = dk / key_parts, part0 = (h % key_parts) * dq;    // the head's own part of a key
+  for (int i = lane; i < dq; i += WAVE) qs[i] = load_f(q, q_dtype, (size_t)r * ldq + (size_t)h * dq + i);
   __syncthreads();
 
   float o[MAX_PER_LANE];
@@ -189,9 +233,9 @@ __global__ __launch_bounds__(64) void masked_attention_plain_kernel(
     const bool valid = t >= first && t <= pos;
     float s = -INFINITY;
     if (valid) {
-      const size_t kb = (size_t)bt[t / P] * page_elems + head_off + (size_t)(t % P) * dk;
+      const size_t kb = (size_t)bt[t / P] * page_elems + head_off + (size_t)(t % P) * dk + part0;
       float dot = 0.f;
-      for (int i = 0; i < dk; ++i) dot = fmaf(qs[i], load_f(cache, cache_dtype, kb + i), dot);
+      for (int i = 0; i < dq; ++i) dot = fmaf(qs[i], load_f(cache, cache_dtype, kb + i), dot);
       s = dot * scale;
     }
     const float m_new = fmaxf(m, wave_max(s));   // finite: every group in the range holds a visible key
@@ -229,15 +273,15 @@ APC_EXPORT int apc_masked_attention_plain(const void* q, int q_dtype, int ldq, v
                                           int n_rows, int H, int G, int dk, int dv, const void* cache, int cache_dtype,
                                           int page_tokens, const int* block_table, int max_blocks,
                                           const int* positions, const int* row_seg, int mask, int mask_size, int sink,
-                                          float scale, hipStream_t stream) {
+                                          float scale, int key_parts, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || page_tokens <= 0 || max_blocks <= 0 || mask < 0 || mask > 2 ||
-      (mask != 0 && mask_size <= 0))
+      (mask != 0 && mask_size <= 0) || key_parts < 1 || dk % key_parts || (H / G) % key_parts)
     return APC_ERR_BAD_ARG;
   if (dk > MAX_PER_LANE * WAVE || dv > MAX_PER_LANE * WAVE || H > 65535) return APC_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(masked_attention_plain_kernel, dim3(n_rows, H), dim3(64), 0, stream, q, q_dtype, ldq, out,
                      out_dtype, ldo, H, G, dk, dv, cache, cache_dtype, page_tokens, block_table, max_blocks, positions,
-                     row_seg, mask, mask_size, sink, scale);
+                     row_seg, mask, mask_size, sink, scale, key_parts);
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -379,11 +379,17 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
                value_dim: int, bias: Optional[torch.Tensor], conv_w: Optional[torch.Tensor],
                state: Optional[torch.Tensor], step, slots: Optional[torch.Tensor], unit_norm: bool, eps: float,
                q_out: torch.Tensor, block_table: Optional[torch.Tensor] = None, cache: Optional[torch.Tensor] = None,
-               page_tokens: int = 0) -> None:
+               page_tokens: int = 0, norm_dim: int = 0, q_norm_w: Optional[torch.Tensor] = None,
+               k_norm_w: Optional[torch.Tensor] = None) -> None:
     """Bias, short causal convolution over time (taps = conv_w.shape[1]; the inputs of the positions ahead of a
     segment come from `state` [slots + 1, taps - 1, width], which is moved on), unit RMS norm of q and k heads,
-    q to `q_out` [rows, heads * key_dim], k and v into the pages.  `n_kv_heads` = 0: the row holds q only."""
-    _gpu(proj, bias, conv_w, state, slots, q_out, block_table, cache)
+    q to `q_out` [rows, heads * key_dim], k and v into the pages.  `n_kv_heads` = 0: the row holds q only.
+    `norm_dim` (divides key_dim; 0: key_dim): the norm is taken over every piece of that many elements of a head;
+    `q_norm_w`, `k_norm_w` float32 [norm_dim]: weights the normed pieces are multiplied with."""
+    _gpu(proj, bias, conv_w, state, slots, q_out, block_table, cache, q_norm_w, k_norm_w)
+    nd = int(norm_dim) or key_dim
+    _need(nd > 0 and key_dim % nd == 0, "conv_heads: norm_dim must divide key_dim")
+    _need((q_norm_w is None and k_norm_w is None) or unit_norm, "conv_heads: norm weights need the norm")
     ld, ldq = _rows(proj, "projected rows"), _rows(q_out, "q out")
     T, width = proj.shape
     G = int(n_kv_heads)
@@ -411,7 +417,8 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
     if (_tuned_ok(proj, q_out) and (cache is None or cache.dtype == torch.bfloat16) and q_off == 0
             and (G == 0 or (k_off == n_heads * key_dim and v_off == (n_heads + G) * key_dim))):
         LT = _lib.load("tuned")
-        if (LT.apc_conv_heads_bf16_takes(ld, width, n_heads, G, key_dim, value_dim, taps, ldq)
+        if (LT.apc_conv_heads_bf16_takes(ld, width, n_heads, G, key_dim, value_dim, taps, ldq) and nd == key_dim
+                and q_norm_w is None and k_norm_w is None
                 and proj.data_ptr() % 16 == 0 and q_out.data_ptr() % 16 == 0
                 and (cache is None or cache.data_ptr() % 16 == 0) and (state is None or state.data_ptr() % 16 == 0)
                 and (conv_w is None or (conv_w.data_ptr() % 16 == 0 and width % 4 == 0))):
@@ -437,7 +444,8 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
         _f32(bias, width, "bias"), _f32(conv_w, width * taps, "conv weights"), taps,
         state.data_ptr() if taps > 1 else 0, width, _i32(step.row_seg, T, "row_seg"), _i32(step.seg_row0, S, "seg_row0"),
         _i32(step.seg_rows, S, "seg_rows"), _i32(slots, S, "slots") if taps > 1 else 0,
-        _i32(step.positions, T, "positions"), 1 if unit_norm else 0, float(eps), q_out.data_ptr(), _code(q_out), ldq,
+        _i32(step.positions, T, "positions"), 1 if unit_norm else 0, float(eps), nd,
+        _f32(q_norm_w, nd, "q norm weight"), _f32(k_norm_w, nd, "k norm weight"), q_out.data_ptr(), _code(q_out), ldq,
         block_table.data_ptr() if G else 0, max_blocks, cache.data_ptr() if G else 0, _code(cache) if G else 0,
         page_tokens, _stream()), "conv_heads")
 
@@ -445,11 +453,12 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
 def masked_attention_plain(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, key_dim: int,
                            value_dim: int, cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor,
                            positions: torch.Tensor, row_seg: torch.Tensor, mask: str, mask_size: int, sink: bool,
-                           scale: float) -> None:
+                           scale: float, key_parts: int = 1) -> None:
     _gpu(q, out, cache, block_table, positions, row_seg)
     ldq, ldo = _rows(q, "attention q"), _rows(out, "attention out")
     T = q.shape[0]
-    _need(q.shape[1] == n_heads * key_dim, "attention: q must be [rows, heads * key_dim]")
+    _check_key_parts(n_heads, n_kv_heads, key_dim, key_parts)
+    _need(q.shape[1] == n_heads * (key_dim // key_parts), "attention: q must be [rows, heads * key_dim / key_parts]")
     _need(out.shape == (T, n_heads * value_dim), "attention out must be [rows, heads * value_dim]")
     _split_pages(cache, n_kv_heads, key_dim, value_dim, page_tokens)
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
@@ -459,19 +468,28 @@ def masked_attention_plain(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_k
         q.data_ptr(), _code(q), ldq, out.data_ptr(), _code(out), ldo, T, n_heads, n_kv_heads, key_dim, value_dim,
         cache.data_ptr(), _code(cache), page_tokens, block_table.data_ptr(), block_table.shape[1],
         _i32(positions, T, "positions"), _i32(row_seg, T, "row_seg"), MASKS[mask], int(mask_size), 1 if sink else 0,
-        float(scale), _stream()), "masked_attention_plain")
+        float(scale), int(key_parts), _stream()), "masked_attention_plain")
+
+
+def _check_key_parts(n_heads: int, n_kv_heads: int, key_dim: int, key_parts: int) -> None:
+    _need(key_parts >= 1 and key_dim % key_parts == 0 and n_heads % n_kv_heads == 0
+          and (n_heads // n_kv_heads) % key_parts == 0,
+          "attention: key_parts must divide key_dim and the query heads of a kv head")
 
 
 def masked_attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int,
                      cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor, step, mask: str = "causal",
-                     mask_size: int = 0, sink: bool = False, scale: float = 1.0) -> None:
-    if _tuned_ok(q, cache, out):
+                     mask_size: int = 0, sink: bool = False, scale: float = 1.0, key_parts: int = 1) -> None:
+    """`key_parts` = M > 1: a cached key of `key_dim` elements is M keys of key_dim / M side by side, one for each of M
+    softmax maps over the same values; q holds `n_heads` heads of key_dim / M, head j uses part j % M (M consecutive
+    heads are the maps of one head), and `out` holds n_heads heads of value_dim (float32 or the run's type)."""
+    if _tuned_ok(q, cache) and out.dtype in (torch.bfloat16, torch.float32):
         from . import tuned
         if tuned.masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens,
-                                       block_table, step, mask, mask_size, sink, scale):
+                                       block_table, step, mask, mask_size, sink, scale, key_parts):
             return
     masked_attention_plain(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens, block_table,
-                           step.positions, step.row_seg, mask, mask_size, sink, scale)
+                           step.positions, step.row_seg, mask, mask_size, sink, scale, key_parts)
 
 
 def streams_step(x: torch.Tensor, n_streams: int, y: Optional[torch.Tensor] = None,
@@ -547,3 +565,155 @@ def scale_(x: torch.Tensor, s: float) -> None:
     _need(x.dtype == torch.float32 and x.is_contiguous(), "scale_: contiguous float32")
     L = _lib.load("plain")
     _lib.check(L.apc_scale(x.data_ptr(), float(s), x.numel(), _stream()), "scale")
+
+
+# --------------------------------------------------------------------------- embedding with positions, normed residual sum
+def embed_positions(table: torch.Tensor, tokens: torch.Tensor, pos_table: torch.Tensor, positions: torch.Tensor,
+                    scale: float, out: torch.Tensor) -> None:
+    """out[t] = table[tokens[t]] * scale + pos_table[positions[t]]  (float32 out; the caller has checked that every
+    position has a row in `pos_table`)."""
+    _gpu(table, tokens, pos_table, positions, out)
+    T = tokens.numel()
+    _need(table.dim() == 2 and table.is_contiguous() and pos_table.dim() == 2 and pos_table.is_contiguous()
+          and pos_table.shape[1] == table.shape[1], "embedding and position tables must be contiguous [n, width]")
+    D = table.shape[1]
+    ldo = _rows(out, "embed out")
+    _need(out.dtype == torch.float32 and out.shape == (T, D), "embed out must be float32 [tokens, width]")
+    L = _lib.load("plain")
+    _lib.check(L.apc_embed_positions(table.data_ptr(), _code(table), _i32(tokens, T, "tokens"), pos_table.data_ptr(),
+                                     _code(pos_table), _i32(positions, T, "positions"), float(scale), out.data_ptr(),
+                                     ldo, T, D, _stream()), "embed_positions")
+
+
+def rmsnorm_add(y: torch.Tensor, weight: torch.Tensor, eps: float, mult: float, x: torch.Tensor,
+                copy: Optional[torch.Tensor] = None, narrow_run: bool = False) -> None:
+    """x += mult * rms_norm(y) * weight, in 32-bit; `copy` (if given) receives the new x in its own element type.
+    `narrow_run`: the step belongs to a bfloat16 run (its kernel library may take the launch)."""
+    _gpu(y, weight, x, copy)
+    ldy, ldx = _rows(y, "rmsnorm_add y"), _rows(x, "rmsnorm_add x")
+    T, D = x.shape
+    _need(x.dtype == torch.float32 and y.shape == (T, D), "rmsnorm_add: x float32 [rows, width], y of the same shape")
+    _need(copy is None or copy.shape == (T, D), "rmsnorm_add: the copy must have x's shape")
+    if narrow_run and not FORCE_PLAIN and y.dtype == torch.float32 and (copy is None or copy.dtype == torch.bfloat16):
+        from . import tuned
+        if tuned.rmsnorm_add_f32(y, weight, eps, mult, x, copy):
+            return
+    L = _lib.load("plain")
+    _lib.check(L.apc_rmsnorm_add(y.data_ptr(), _code(y), ldy, _f32(weight, D, "norm weight"), float(eps), float(mult),
+                                 x.data_ptr(), ldx, copy.data_ptr() if copy is not None else 0,
+                                 _code(copy) if copy is not None else 0,
+                                 _rows(copy, "rmsnorm_add copy") if copy is not None else 0, T, D, _stream()),
+               "rmsnorm_add")
+
+
+# --------------------------------------------------------------------------- linear attention with a decay
+def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: int, key_dim: int,
+                     value_dim: int, silu: bool, decay: torch.Tensor, state: torch.Tensor, step, slots: torch.Tensor,
+                     out: torch.Tensor) -> None:
+    """Per head S <- decay * S + k_t v_t^T, o_t = S^T q_t over the rows of every segment in order, S float32
+    [slots + 1, heads, key_dim, value_dim] per request; q, k, v (through silu if asked) from the projected rows;
+    `out` float32 [rows, heads * value_dim]."""
+    _gpu(proj, decay, state, slots, out)
+    ld, ldo = _rows(proj, "projected rows"), _rows(out, "linear attention out")
+    T, width = proj.shape
+    H, dk, dv = int(n_heads), int(key_dim), int(value_dim)
+    _need(q_off + H * dk <= width and k_off + H * dk <= width and v_off + H * dv <= width,
+          "linear attention: head ranges exceed the row")
+    _need(out.dtype == torch.float32 and out.shape == (T, H * dv), "linear attention: out float32 [rows, heads * value_dim]")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, dk, dv),
+          f"linear attention: state must be float32 [slots, {H}, {dk}, {dv}]")
+    S = step.n_segs
+    if _tuned_ok(proj):
+        from . import tuned
+        if tuned.linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, state, step, slots, out):
+            return
+    L = _lib.load("plain")
+    _lib.check(L.apc_linear_attention(proj.data_ptr(), _code(proj), ld, q_off, k_off, v_off, H, dk, dv,
+                                      1 if silu else 0, _f32(decay, H, "decay"), state.data_ptr(), S,
+                                      _i32(step.seg_row0, S, "seg_row0"), _i32(step.seg_rows, S, "seg_rows"),
+                                      _i32(slots, S, "slots"), out.data_ptr(), ldo, _stream()), "linear_attention")
+
+
+def gated_rmsnorm(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: Optional[torch.Tensor],
+                  out: torch.Tensor) -> None:
+    """out = rms_norm(o) * weight * sigmoid(gate), the norm over the whole row; o float32, gate (logits) and out any."""
+    _gpu(o, weight, gate, out)
+    T, N = o.shape
+    _need(o.dtype == torch.float32 and out.shape == (T, N) and (gate is None or gate.shape == (T, N)),
+          "gated_rmsnorm: o float32 [rows, n], gate and out of the same shape")
+    L = _lib.load("plain")
+    _lib.check(L.apc_gated_rmsnorm(o.data_ptr(), _rows(o, "o"), _f32(weight, N, "norm weight"), float(eps),
+                                   gate.data_ptr() if gate is not None else 0, _code(gate) if gate is not None else 0,
+                                   _rows(gate, "gate") if gate is not None else 0, out.data_ptr(), _code(out),
+                                   _rows(out, "out"), T, N, _stream()), "gated_rmsnorm")
+
+
+def diff_combine(a: torch.Tensor, lam: float, post: float, eps: float, gate: Optional[torch.Tensor],
+                 out: torch.Tensor, n_heads: int, value_dim: int) -> None:
+    """a float32 [rows, heads * 2 * value_dim] (per head: map 1, map 2): o = a1 - lam * a2, divided by its root mean
+    square over the head, times `post` and sigmoid(gate[row][head]) (gate logits [rows, heads], or None)."""
+    _gpu(a, gate, out)
+    T = a.shape[0]
+    H, dv = int(n_heads), int(value_dim)
+    _need(a.dtype == torch.float32 and a.shape == (T, 2 * H * dv) and out.shape == (T, H * dv),
+          "diff_combine: a float32 [rows, heads * 2 * value_dim], out [rows, heads * value_dim]")
+    _need(gate is None or gate.shape == (T, H), "diff_combine: gate must be [rows, heads]")
+    L = _lib.load("plain")
+    _lib.check(L.apc_diff_combine(a.data_ptr(), _rows(a, "a"), float(lam), float(post), float(eps),
+                                  gate.data_ptr() if gate is not None else 0, _code(gate) if gate is not None else 0,
+                                  _rows(gate, "gate") if gate is not None else 0, out.data_ptr(), _code(out),
+                                  _rows(out, "out"), T, H, dv, _stream()), "diff_combine")
+
+
+# --------------------------------------------------------------------------- routed experts
+def route_topk(z: torch.Tensor, correction: Optional[torch.Tensor], top: int, ids: torch.Tensor,
+               weights: torch.Tensor, renormalize: bool = False) -> None:
+    """s = softmax(z) over a row; the `top` largest of s + correction are chosen (the lower index wins a tie);
+    weights = s of the chosen (divided by their sum with `renormalize`).  z float32 [rows, n]."""
+    _gpu(z, correction, ids, weights)
+    T, N = z.shape
+    _need(z.dtype == torch.float32 and weights.dtype == torch.float32 and weights.is_contiguous()
+          and weights.numel() >= T * top, "route_topk: z float32, weights contiguous float32 [rows, top]")
+    L = _lib.load("plain")
+    _lib.check(L.apc_route_topk(z.data_ptr(), _rows(z, "router logits"), _f32(correction, N, "correction"), T, N,
+                                int(top), 1 if renormalize else 0, _i32(ids, T * top, "ids"), weights.data_ptr(),
+                                _stream()), "route_topk")
+
+
+def prepare_experts(gate_up: torch.Tensor, down: torch.Tensor, run_dtype: torch.dtype):
+    """How the experts' matrices [experts, 2 ff, width] and [experts, width, ff] are kept on the GPU: in the tiled
+    layout of the MFMA kernels for a bfloat16 run whose sizes they take, else as they are."""
+    if run_dtype == torch.bfloat16 and not FORCE_PLAIN and gate_up.is_cuda and gate_up.dtype == torch.bfloat16:
+        from . import tuned
+        packed = tuned.pack_experts(gate_up, down)
+        if packed is not None:
+            return packed
+    return gate_up.contiguous(), down.contiguous()
+
+
+def routed_experts(h: torch.Tensor, w_gate_up, w_down, n_experts: int, ff: int, ids: torch.Tensor,
+                   weights: torch.Tensor, top: int, y: torch.Tensor) -> None:
+    """y[t] = sum_k weights[t][k] * expert ids[t][k] (h[t]); experts 0 .. n_experts-1 are gated units
+    Wd (silu(Wg h) * (Wu h)) with w_gate_up [n_experts, 2 * ff, width] (gate rows, then up rows) and w_down
+    [n_experts, width, ff]; ids from n_experts on are identity experts.  y float32 [rows, width]."""
+    T, D = h.shape
+    E, F, K = int(n_experts), int(ff), int(top)
+    _gpu(h, ids, weights, y)
+    _need(y.dtype == torch.float32 and y.shape == (T, D), "routed_experts: y float32 [rows, width]")
+    if not isinstance(w_gate_up, torch.Tensor) and w_gate_up is not None:
+        from . import tuned
+        tuned.routed_experts_bf16(h, w_gate_up, w_down, E, F, ids, weights, K, y)
+        return
+    act = torch.empty((T * K, F), dtype=h.dtype, device=h.device)
+    L = _lib.load("plain")
+    if E:
+        _gpu(w_gate_up, w_down)
+        _need(w_gate_up.is_contiguous() and tuple(w_gate_up.shape) == (E, 2 * F, D) and w_down.is_contiguous()
+              and tuple(w_down.shape) == (E, D, F), "routed_experts: matrices [experts, 2 ff, width] and [experts, width, ff]")
+        _lib.check(L.apc_routed_glu(h.data_ptr(), _code(h), _rows(h, "h"), w_gate_up.data_ptr(), _code(w_gate_up), E, F,
+                                    D, _i32(ids, T * K, "ids"), K, act.data_ptr(), _code(act), T, _stream()),
+                   "routed_glu")
+    _lib.check(L.apc_routed_down(act.data_ptr(), _code(act), w_down.data_ptr() if E else 0,
+                                 _code(w_down) if E else 0, E, F, D, _i32(ids, T * K, "ids"),
+                                 _f32(weights, T * K, "weights"), K, h.data_ptr(), _code(h), _rows(h, "h"),
+                                 y.data_ptr(), _rows(y, "y"), T, _stream()), "routed_down")

@@ -461,7 +461,7 @@ MASKED_DECODE_SPLITS = 64     # at most: the adding kernel takes 64 parts
 
 
 def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens, block_table, step,
-                          mask: str, mask_size: int, sink: bool, scale: float) -> bool:
+                          mask: str, mask_size: int, sink: bool, scale: float, key_parts: int = 1) -> bool:
     """Attention with a chunked or sliding mask and an optional sink on the MFMA kernels: segments of several rows on
     the tiled kernel, single rows on the kernel that cuts a row's keys into ranges.  False (nothing done) for sizes
     they do not take; the caller then runs the plain kernel."""
@@ -469,6 +469,8 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
     ldq, ldo = _ops._rows(q, "attention q"), _ops._rows(out, "attention out")
     T = q.shape[0]
     L = _lib.load("tuned")
+    if key_parts != 1:
+        return False
     if (not scale > 0 or ldq % 8 or ldo % 4 or not _aligned(q, cache) or out.data_ptr() % 8
             or q.dtype != torch.bfloat16 or cache.dtype != torch.bfloat16 or out.dtype != torch.bfloat16
             or not L.apc_attention_masked_takes(n_heads, n_kv_heads, key_dim, value_dim, page_tokens)):
@@ -499,3 +501,15 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
             int(mask_size), 1 if sink else 0, float(scale), splits, parts.data_ptr(), stream),
             "attention_masked_decode_bf16")
     return True
+
+
+def rmsnorm_add_f32(y, weight, eps, mult, x, copy) -> bool:
+    return False
+
+
+def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, state, step, slots, out) -> bool:
+    return False
+
+
+def pack_experts(gate_up, down):
+    return None

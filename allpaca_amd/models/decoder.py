@@ -87,7 +87,10 @@ class DecoderModel:
         with several residual streams)."""
         x = torch.empty((step.n_rows, self.spec.streams * self.spec.hidden_size), dtype=torch.float32,
                         device=self.rt.device)
-        self.embedding.forward(step.tokens, x)
+        if getattr(self.embedding, "reads_positions", False):
+            self.embedding.forward_step(step, x)
+        else:
+            self.embedding.forward(step.tokens, x)
         return x
 
     def run_plan(self, x: torch.Tensor, step, caches, lo: int, hi: int, left):

@@ -174,3 +174,63 @@ class HyperPreNorm:
             return StreamsLeft(next_norm.connection, next_norm.norm, h)
         last.write(x, y)
         return None
+
+
+class RowsLeft:
+    """What a layer whose sublayers read the residual itself leaves for the next one: the residual in the run's
+    element type (the kernel that adds the last sublayer's output writes it on the way)."""
+
+    def __init__(self, h: torch.Tensor):
+        self.h = h
+
+
+class ReadsResidual:
+    """What such a layer shows the layer before it: its first sublayer reads the residual as it is."""
+
+    def rms_params(self):       # to an arrangement that folds norms into products this is no norm it can fold
+        return None
+
+
+@ARRANGEMENTS.register("sublayer_norm")
+class SublayerNorm:
+    """The norm stands on the sublayer's output only, and the sum is scaled:
+       x <- x + mult * norm1(mixer(x));  x <- x + mult * norm2(ffn(x))      (a layer may have no feed-forward)
+    The sublayers read x itself (in the run's element type).  Norm and sum are one kernel in 32-bit, which also
+    leaves the new x in the run's element type for the next sublayer."""
+    registries = {"mixer": MIXERS, "mixer_norm": NORMS, "ffn": FEED_FORWARDS, "ffn_norm": NORMS, "scale": CONNECTIONS}
+    chains_norms = True
+
+    @staticmethod
+    def first_norm(parts):
+        return ReadsResidual()
+
+    @staticmethod
+    def run(parts, x: torch.Tensor, step, cache, pre=None, next_norm=None):
+        from ..kernels import ops
+        mixer, ffn = parts["mixer"], parts.get("ffn")
+        rt = mixer.rt
+        mult = parts["scale"].mult
+        narrow = rt.dtype != torch.float32       # a 32-bit run reads x as it is: no copy
+
+        def copy():
+            return torch.empty(x.shape, dtype=rt.dtype, device=x.device) if narrow else None
+
+        if not narrow:
+            h = x
+        elif isinstance(pre, RowsLeft):
+            h = pre.h
+        else:
+            h = copy()
+            ops.cast(x, h)
+        y = mixer.forward(h, step, cache)
+        w, eps = parts["mixer_norm"].rms_params()
+        last = ffn is None
+        wants = isinstance(next_norm, ReadsResidual)
+        h = copy() if (not last or wants) else None
+        ops.rmsnorm_add(y, w, eps, mult, x, h, narrow_run=narrow)
+        if not last:
+            y = ffn.forward(h if narrow else x, step)
+            w, eps = parts["ffn_norm"].rms_params()
+            h = copy() if wants else None
+            ops.rmsnorm_add(y, w, eps, mult, x, h, narrow_run=narrow)
+        return RowsLeft(h) if (wants and narrow) else None

@@ -55,3 +55,12 @@ class HyperConnection(Part):
             return
         w, eps = norm.rms_params()
         ops.streams_step(x, self.S, y=y, mix=self.w_mix, out_w=self.w_out, in_w=then.w_in, norm_w=w, eps=eps, h=h)
+
+
+@CONNECTIONS.register("scaled")
+class ScaledSum(Part):
+    """x <- x + mult * y: a constant of the layer, no tensors."""
+    graph_safe = True
+
+    def __init__(self, mult: float = 1.0):
+        self.mult = float(mult)

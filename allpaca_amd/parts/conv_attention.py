@@ -11,7 +11,12 @@ Per row, with h the mixer's input:
 Keys have `key_dim` and values `value_dim` elements a head; query head j reads kv head j // (H / G).  The cache holds
 k after convolution and norm and v after convolution.  With `shares_kv` the mixer has no k and v of its own: it reads
 the pages of the plan entry it borrows from (`PlanEntry.cache_of`) with its own q.  The projected rows of the last
-taps - 1 positions are per-request state (float32), kept by the mixer itself also when it borrows."""
+taps - 1 positions are per-request state (float32), kept by the mixer itself also when it borrows.
+
+`key_parts` = M > 1: a head has M softmax maps over the same values.  `key_dim` then counts all M queries (keys) of a
+head side by side, the unit norm is taken over each of the M pieces, and `attend` returns the M maps' outputs of every
+head side by side in float32 for a subclass to combine (`DifferentialAttention`).  `norm_weights`: the normed pieces of
+q and k are multiplied with the tensors "<q>.norm" and "<k>.norm" [key_dim / M], shared by all heads and maps."""
 from __future__ import annotations
 
 from typing import Dict, Mapping, Optional
@@ -30,7 +35,8 @@ class ConvAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int,
                  scale: float, conv_taps: int = 0, unit_norm: bool = True, norm_eps: float = 1e-6, bias: bool = True,
                  mask: str = "causal", mask_size: int = 0, sink: bool = False, shares_kv: bool = False,
-                 names: Optional[Mapping[str, str]] = None):
+                 names: Optional[Mapping[str, str]] = None, key_parts: int = 1, norm_weights: bool = False,
+                 extra_rows: int = 0):
         if num_heads % num_kv_heads:
             raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         if mask not in ops.MASKS or (mask != "causal" and int(mask_size) <= 0):
@@ -42,8 +48,13 @@ class ConvAttention(Mixer):
         self.unit_norm, self.eps, self.bias = bool(unit_norm), float(norm_eps), bool(bias)
         self.mask, self.mask_size, self.sink = mask, int(mask_size), bool(sink)
         self.shares_kv = bool(shares_kv)
+        self.key_parts, self.norm_weights = int(key_parts), bool(norm_weights)
+        if self.key_parts < 1 or self.dk % self.key_parts or (self.norm_weights and not self.unit_norm):
+            raise ValueError(f"attention: key_parts {key_parts} must divide key_dim {key_dim}, and norm weights need the norm")
+        self.extra_rows = int(extra_rows)      # rows a subclass adds to the input matrix behind q, k and v
         # tensor names: projections q, k, v, o; "<projection><bias>" and "<projection><conv>" beside them
-        self.names = {"q": "q", "k": "k", "v": "v", "o": "o", "bias": ".b", "conv": ".conv", **dict(names or {})}
+        self.names = {"q": "q", "k": "k", "v": "v", "o": "o", "bias": ".b", "conv": ".conv", "norm": ".norm",
+                      **dict(names or {})}
         self.projections = [("q", self.H * self.dk)]
         if not self.shares_kv:
             self.projections += [("k", self.G * self.dk), ("v", self.G * self.dv)]
@@ -59,8 +70,15 @@ class ConvAttention(Mixer):
                 out[n[p] + n["bias"]] = ParamSpec((rows,), store="float32", init="zeros")
             if self.taps >= 1:
                 out[n[p] + n["conv"]] = ParamSpec((rows, self.taps), store="float32", init="normal")
+        if self.norm_weights:
+            for p, _ in self.projections[:2]:
+                out[n[p] + n["norm"]] = ParamSpec((self.dk // self.key_parts,), store="float32")
         out[n["o"]] = ParamSpec((self.D, self.H * self.dv))
         return out
+
+    def extra_matrices(self, tensors, rt) -> list:
+        """Matrices [rows, hidden] of a subclass that go into the one input product behind q, k and v."""
+        return []
 
     def cache_need(self):
         return None if self.shares_kv else PagedKeysValues(self.G, self.dk, self.dv)
@@ -71,8 +89,13 @@ class ConvAttention(Mixer):
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
         self.rt = rt
         n = self.names
-        mats = [tensors[n[p]] for p, _ in self.projections]
+        mats = [tensors[n[p]] for p, _ in self.projections] + list(self.extra_matrices(tensors, rt))
         dt = mats[0].dtype if all(m.dtype == mats[0].dtype for m in mats) else torch.float32
+        self.q_norm_w = self.k_norm_w = None
+        if self.norm_weights:
+            self.q_norm_w = to_device(tensors[n["q"] + n["norm"]], rt, torch.float32)
+            if not self.shares_kv:
+                self.k_norm_w = to_device(tensors[n["k"] + n["norm"]], rt, torch.float32)
         # one [width, D] matrix: a single product gives q (, k and v) of a row
         self.w_in = ops.prepare_matrix(torch.cat([to_device(m, rt, dt) for m in mats], dim=0), rt.dtype)
         self.w_o = ops.prepare_matrix(to_device(tensors[n["o"]], rt), rt.dtype)
@@ -84,14 +107,16 @@ class ConvAttention(Mixer):
             self.conv_w = torch.cat([to_device(tensors[n[p] + n["conv"]], rt, torch.float32)
                                      for p, _ in self.projections], dim=0).contiguous()
 
-    def forward(self, h, step, cache) -> torch.Tensor:
-        """float32 [rows, hidden]: the mixer's output.  `cache`: the pages' view, or {"mixer": pages,
+    def attend(self, h, step, cache, out_dtype=None):
+        """(the input product's rows [rows, width + extra_rows], the attention's output [rows, heads * key_parts *
+        value_dim] in `out_dtype`, the run's type if None).  `cache`: the pages' view, or {"mixer": pages,
         "mixer.state": the convolution's state}."""
         pages, state = (cache.get("mixer"), cache.get("mixer.state")) if isinstance(cache, dict) else (cache, None)
         h = as_normed(h).tensor()
         T, dev, dt = h.shape[0], h.device, self.rt.dtype
-        proj = torch.empty((T, self.width), dtype=dt, device=dev)
-        ops.linear(h, self.w_in, proj)
+        full = torch.empty((T, self.width + self.extra_rows), dtype=dt, device=dev)
+        ops.linear(h, self.w_in, full)
+        proj = full[:, :self.width] if self.extra_rows else full
         q = torch.empty((T, self.H * self.dk), dtype=dt, device=dev)
         own = not self.shares_kv
         if own and not pages.writes:
@@ -99,10 +124,70 @@ class ConvAttention(Mixer):
         ops.conv_heads(proj, self.q_off, self.k_off, self.v_off, self.H, self.G if own else 0, self.dk, self.dv,
                        self.b_in, self.conv_w, state.state if state is not None else None, step,
                        state.slots if state is not None else None, self.unit_norm, self.eps, q,
-                       pages.block_table if own else None, pages.kv if own else None, pages.page_tokens)
-        attn = torch.empty((T, self.H * self.dv), dtype=dt, device=dev)
-        ops.masked_attention(q, attn, self.H, self.G, self.dk, self.dv, pages.kv, pages.page_tokens,
-                             pages.block_table, step, self.mask, self.mask_size, self.sink, self.scale)
+                       pages.block_table if own else None, pages.kv if own else None, pages.page_tokens,
+                       norm_dim=self.dk // self.key_parts, q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w)
+        M = self.key_parts
+        attn = torch.empty((T, self.H * M * self.dv), dtype=out_dtype or dt, device=dev)
+        ops.masked_attention(q, attn, self.H * M, self.G, self.dk, self.dv, pages.kv, pages.page_tokens,
+                             pages.block_table, step, self.mask, self.mask_size, self.sink, self.scale, key_parts=M)
+        return full, attn
+
+    def forward(self, h, step, cache) -> torch.Tensor:
+        """float32 [rows, hidden]: the mixer's output."""
+        if self.key_parts != 1:
+            raise ValueError("an attention with several maps a head needs a rule that combines them")
+        _, attn = self.attend(h, step, cache)
+        T, dev = attn.shape[0], attn.device
+        out = torch.empty((T, self.D), dtype=torch.float32, device=dev)
+        ops.linear(attn, self.w_o, out)
+        return out
+
+
+@MIXERS.register("differential_attention")
+class DifferentialAttention(ConvAttention):
+    """Two softmax maps a head over the same values, a1 and a2:
+      lam = exp(lq1 . lk1) - exp(lq2 . lk2) + diff            (one number for the layer)
+      o = a1 - lam * a2;  o <- o / sqrt(mean(o^2) + eps) over the head's values, times (1 - diff)
+      o <- o * sigmoid(Wg h)[head]  (`head_gate`: one number a head, from the mixer's input);  out = Wo o
+    q holds [map 1, map 2] of `key_dim` each per head, k likewise per kv head; convolution, norm (with weights), mask
+    and pages are the base class's."""
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, scale: float,
+                 diff: float, conv_taps: int = 0, norm_eps: float = 1e-6, head_gate: bool = True,
+                 shares_kv: bool = False, mask: str = "causal", mask_size: int = 0,
+                 names: Optional[Mapping[str, str]] = None):
+        names = {"lq1": "lq1", "lk1": "lk1", "lq2": "lq2", "lk2": "lk2", "gate": "g", **dict(names or {})}
+        super().__init__(hidden_size, num_heads, num_kv_heads, 2 * int(key_dim), value_dim, scale, conv_taps=conv_taps,
+                         unit_norm=True, norm_eps=norm_eps, bias=False, mask=mask, mask_size=mask_size, sink=False,
+                         shares_kv=shares_kv, names=names, key_parts=2, norm_weights=True,
+                         extra_rows=int(num_heads) if head_gate else 0)
+        self.diff, self.head_gate, self.map_dim = float(diff), bool(head_gate), int(key_dim)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        out = super().param_specs()
+        n = self.names
+        for x in ("lq1", "lk1", "lq2", "lk2"):
+            out[n[x]] = ParamSpec((self.map_dim,), store="float32", init="normal")
+        if self.head_gate:
+            out[n["gate"]] = ParamSpec((self.H, self.D))
+        return out
+
+    def extra_matrices(self, tensors, rt) -> list:
+        return [tensors[self.names["gate"]]] if self.head_gate else []
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        super().bind(tensors, rt)
+        n = self.names
+        lq1, lk1, lq2, lk2 = (tensors[n[x]].to(torch.float32) for x in ("lq1", "lk1", "lq2", "lk2"))
+        self.lam = float(torch.exp(torch.dot(lq1, lk1)) - torch.exp(torch.dot(lq2, lk2))) + self.diff
+
+    def forward(self, h, step, cache) -> torch.Tensor:
+        full, maps = self.attend(h, step, cache, out_dtype=torch.float32)
+        T, dev = maps.shape[0], maps.device
+        attn = torch.empty((T, self.H * self.dv), dtype=self.rt.dtype, device=dev)
+        gate = full[:, self.width:self.width + self.H] if self.head_gate else None
+        ops.diff_combine(maps, self.lam, 1.0 - self.diff, self.eps, gate, attn, self.H, self.dv)
         out = torch.empty((T, self.D), dtype=torch.float32, device=dev)
         ops.linear(attn, self.w_o, out)
         return out

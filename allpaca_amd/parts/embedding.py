@@ -56,6 +56,34 @@ class NormedTokenEmbedding(Part):
         ops.embed_streams(self.weight, tokens, self.norm_weight, self.eps, out, self.S)
 
 
+@EMBEDDINGS.register("token_table_positions")
+class PositionedTokenEmbedding(Part):
+    """A token's row of the table times `scale`, plus a learned vector of the token's position (not scaled):
+    x = table[token] * scale + positions[p].  The position table has `max_positions` rows; a step that reaches
+    beyond them is refused."""
+    graph_safe = True
+    reads_positions = True       # `forward_step(step, out)` instead of `forward(tokens, out)`
+
+    def __init__(self, vocab_size: int, hidden_size: int, max_positions: int, scale: float = 1.0,
+                 table_name: str = "weight", positions_name: str = "positions"):
+        self.V, self.D, self.P, self.scale = int(vocab_size), int(hidden_size), int(max_positions), float(scale)
+        self.table_name, self.positions_name = table_name, positions_name
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {self.table_name: ParamSpec((self.V, self.D)), self.positions_name: ParamSpec((self.P, self.D))}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+        self.weight = to_device(tensors[self.table_name], rt)      # row-major: rows are read whole
+        self.positions = to_device(tensors[self.positions_name], rt)
+
+    def forward_step(self, step, out: torch.Tensor) -> None:
+        if step.max_context > self.P:
+            raise ValueError(f"a request reaches position {step.max_context - 1}, the model has position vectors for "
+                             f"{self.P} positions")
+        ops.embed_positions(self.weight, step.tokens, self.positions, step.positions, self.scale, out)
+
+
 @HEADS.register("linear")
 class LinearHead(Part):
     """`tied`: the head uses the embedding matrix and owns no tensor."""

@@ -19,19 +19,23 @@ class SwiGLU(FeedForward):
     takes_normed_input = True
     emits_next_norm = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    def __init__(self, hidden_size: int, intermediate_size: int, names: Mapping[str, str] | None = None):
         self.D, self.F = int(hidden_size), int(intermediate_size)
+        # tensor names of the three matrices
+        self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight",
+                      **dict(names or {})}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
+        n = self.names
         return {
-            "gate_proj.weight": ParamSpec((self.F, self.D)),
-            "up_proj.weight": ParamSpec((self.F, self.D)),
-            "down_proj.weight": ParamSpec((self.D, self.F)),
+            n["gate"]: ParamSpec((self.F, self.D)),
+            n["up"]: ParamSpec((self.F, self.D)),
+            n["down"]: ParamSpec((self.D, self.F)),
         }
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
         self.rt = rt
-        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
         dt = g.dtype if g.dtype == u.dtype else torch.float32
         # one pass over h gives both branches: the pair of tiled matrices for the MFMA kernels, else
         # [2F, D] (gate rows, then up rows)
@@ -40,7 +44,7 @@ class SwiGLU(FeedForward):
             self.w_gate_up = torch.cat([wg, wu], dim=0).contiguous()
         else:
             self.w_gate_up = (wg, wu)
-        self.w_down = ops.prepare_matrix(to_device(tensors["down_proj.weight"], rt), rt.dtype)
+        self.w_down = ops.prepare_matrix(to_device(tensors[self.names["down"]], rt), rt.dtype)
 
     def forward_add(self, h, step, residual: torch.Tensor, emit=None) -> None:
         h = as_normed(h)
@@ -54,8 +58,11 @@ class SwiGLU(FeedForward):
         return {"kind": "swiglu", "w_gate_up": self.w_gate_up, "w_down": self.w_down, "F": self.F}
 
     def forward(self, h, step):
-        out = torch.zeros((h.shape[0], self.D), dtype=torch.float32, device=h.device)
-        self.forward_add(h, step, out)
+        h = as_normed(h)
+        act = torch.empty((h.shape[0], self.F), dtype=self.rt.dtype, device=h.device)
+        h.swiglu(self.w_gate_up, act)
+        out = torch.empty((h.shape[0], self.D), dtype=torch.float32, device=h.device)
+        ops.linear(act, self.w_down, out)
         return out
 
 
