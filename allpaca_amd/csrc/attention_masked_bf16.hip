@@ -5,6 +5,11 @@
 //   n positions counted from position 0);  s = (q . k) * scale;  weights exp(s) / (sink + sum exp(s)), sink = 1 (a key
 //   of score 0 without a value) or 0;  query head h reads kv head h / (H / G).
 //
+// `key_parts` = M > 1: a cached key of dk elements is M keys of dk / M side by side, one for each of M softmax maps over
+// the same values; q holds H heads of dk / M, head j uses part j % M of the keys (M consecutive heads are the maps of
+// one head).  The kernels keep the whole key as the summed axis and give a head's query zeros outside its own part, so
+// nothing else changes; `out_f32`: the heads' outputs leave in float32 (for a caller that combines the maps).
+//
 // Pages: one row per kv head, first the page's keys [slot][dk], then its values [dv][slot]; a page is
 // G * P * (dk + dv) elements.
 //
@@ -53,10 +58,11 @@ __device__ __forceinline__ float exp2_neg(float x) { return __builtin_amdgcn_exp
 // ------------------------------------------------------------------------------------------ prompt portions
 template <int DKP, int DVP>  // key and value sizes rounded up to a multiple of 32
 __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
-    const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, int H, int G, int dk, int dv,
+    const bf16_t* __restrict__ q, int ldq, void* __restrict__ out, int ldo, int H, int G, int dk, int dv,
     const bf16_t* __restrict__ cache, int P, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
-    const int* __restrict__ tile_rows, int n_tiles, int mask, int mask_size, int sink, float scale) {
+    const int* __restrict__ tile_rows, int n_tiles, int mask, int mask_size, int sink, float scale, int key_parts,
+    int out_f32) {
   constexpr int KROW = DKP + (DKP % 128 == 0 ? 72 : DKP % 128 == 64 ? 8 : DKP % 128 == 32 ? 40 : 104);
   __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KROW];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[DVP * (KT + KPAD)];
@@ -95,11 +101,12 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
   const int my_row = wave * 16 + li;
   Frag qf[DKP / 32];
   {
-    const bf16_t* qrow = q + (size_t)(row0 + min(my_row, nrows - 1)) * ldq + (size_t)h * dk;
+    const int dq = dk / key_parts, part0 = (h % key_parts) * dq;     // the head's own part of a key
+    const bf16_t* qrow = q + (size_t)(row0 + min(my_row, nrows - 1)) * ldq + (size_t)h * dq;
 #pragma unroll
     for (int ks = 0; ks < DKP / 32; ++ks) {
       const int e = ks * 32 + lc * 8;
-      qf[ks] = (my_row < nrows && e < dk) ? load_frag(qrow + e) : zero_frag();
+      qf[ks] = (my_row < nrows && e >= part0 && e < part0 + dq) ? load_frag(qrow + (e - part0)) : zero_frag();
     }
   }
   const int my_pos = pos0 + my_row;
@@ -244,11 +251,15 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
   }
   if (my_row < nrows) {
     const float inv = 1.0f / l_run;
-    bf16_t* orow = out + (size_t)(row0 + my_row) * ldo + (size_t)h * dv;
+    const size_t at = (size_t)(row0 + my_row) * ldo + (size_t)h * dv;
+    bf16_t* orow = (bf16_t*)out + at;
 #pragma unroll
     for (int dt = 0; dt < DVP / 16; ++dt) {
       const int e = dt * 16 + lc * 4;
-      if (e < dv) {
+      if (e < dv && out_f32) {
+        *reinterpret_cast<float4*>((float*)out + at + e) =
+            float4{o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv};
+      } else if (e < dv) {
         uint2 pk;
         pk.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
         pk.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
@@ -281,7 +292,7 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     const bf16_t* __restrict__ q, int ldq, int H, int G, int dk, int dv, const bf16_t* __restrict__ cache, int P,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ positions,
     const int* __restrict__ row_seg, const int* __restrict__ rows, int mask, int mask_size, float scale, int n_splits,
-    float* __restrict__ parts) {
+    float* __restrict__ parts, int key_parts) {
   __shared__ __attribute__((aligned(16))) float sc_all[NW][HGMAX * SROW];
   __shared__ __attribute__((aligned(16))) bf16_t ps_all[NW][HGMAX * PROW];
   __shared__ float ml_all[NW][HGMAX][3];        // running maximum, running sum, the last pass's factor
@@ -302,10 +313,12 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
 
   // the heads' queries as the second operand: column li = head, 8 elements from (ks * 32 + lc * 8) on
   Frag qf[KS];
+  const int dq = dk / key_parts, part0 = (li % key_parts) * dq;      // (per is a multiple of key_parts)
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     const int c = ks * 32 + lc * 8;
-    qf[ks] = (li < per && c < dk) ? load_frag(q + (size_t)r * ldq + (size_t)(g * per + li) * dk + c) : zero_frag();
+    qf[ks] = (li < per && c >= part0 && c < part0 + dq)
+                 ? load_frag(q + (size_t)r * ldq + (size_t)(g * per + li) * dq + (c - part0)) : zero_frag();
   }
   for (int idx = lane; idx < HGMAX * PROW; idx += WAVE) ps[idx] = 0;    // rows of heads that do not exist stay 0
   if (lane < HGMAX) { ml[lane][0] = -INFINITY; ml[lane][1] = 0.f; ml[lane][2] = 1.f; }
@@ -430,7 +443,7 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
 // no condition on the way (a part beyond the last one is read as the last one, with weight 0).
 __global__ __launch_bounds__(64) void attn_masked_merge_kernel(const float* __restrict__ parts, int n_parts, int H,
                                                                int dv, const int* __restrict__ rows, int sink,
-                                                               bf16_t* __restrict__ out, int ldo) {
+                                                               void* __restrict__ out, int ldo, int out_f32) {
   const int ri = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = rows ? rows[ri] : ri;
   const float* p = parts + ((size_t)ri * H + h) * n_parts * (dv + 2);
@@ -451,18 +464,19 @@ __global__ __launch_bounds__(64) void attn_masked_merge_kernel(const float* __re
 #pragma unroll
       for (int k = 0; k < 16; ++k) a = fmaf(s0 + k < n_parts ? __shfl(w, (s0 + k) & 63, WAVE) : 0.f, v[k], a);
     }
-    if (e0 + lane < dv) out[(size_t)r * ldo + (size_t)h * dv + e] = float_to_bf16(a * inv);
+    if (e0 + lane < dv) store_f(out, out_f32 ? APC_F32 : APC_BF16, (size_t)r * ldo + (size_t)h * dv + e, a * inv);
   }
 }
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 int check_sizes(const void* q, int ldq, const void* out, int ldo, const void* cache, int H, int G, int dk, int dv, int P,
-                int mask, int mask_size, float scale) {
-  if (H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || P <= 0 || mask < 0 || mask > 2 || (mask && mask_size <= 0))
+                int mask, int mask_size, float scale, int key_parts, int out_f32) {
+  if (H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || P <= 0 || mask < 0 || mask > 2 || (mask && mask_size <= 0) ||
+      key_parts < 1 || dk % key_parts || (H / G) % key_parts)
     return APC_ERR_BAD_ARG;
-  if (dk % 8 || dv % 4 || dk > DMAX || dv > DMAX || P % 8 || ldq % 8 || ldo % 4 || !aligned16(q) || !aligned16(cache) ||
-      ((uintptr_t)out & 7u) || !(scale > 0.f))
+  if (dk % (8 * key_parts) || dv % 4 || dk > DMAX || dv > DMAX || P % 8 || ldq % 8 || ldo % 4 || !aligned16(q) ||
+      !aligned16(cache) || ((uintptr_t)out & (out_f32 ? 15u : 7u)) || !(scale > 0.f))
     return APC_ERR_UNSUPPORTED;
   return 0;
 }
@@ -470,9 +484,9 @@ int check_sizes(const void* q, int ldq, const void* out, int ldo, const void* ca
 }  // namespace
 
 // 1 if the kernels take these sizes, else 0 (the caller then runs the plain kernel)
-APC_EXPORT int apc_attention_masked_takes(int H, int G, int dk, int dv, int page_tokens) {
-  if (H <= 0 || G <= 0 || H % G || H / G > 16) return 0;
-  if (dk % 8 || dv % 8 || dk > DMAX || dv > DMAX) return 0;
+APC_EXPORT int apc_attention_masked_takes(int H, int G, int dk, int dv, int page_tokens, int key_parts) {
+  if (H <= 0 || G <= 0 || H % G || H / G > 16 || key_parts < 1 || (H / G) % key_parts) return 0;
+  if (dk % (8 * key_parts) || dv % 8 || dk > DMAX || dv > DMAX) return 0;
   if (page_tokens < 8 || page_tokens > DT || (page_tokens & (page_tokens - 1))) return 0;
   return 1;
 }
@@ -481,17 +495,19 @@ APC_EXPORT int apc_attention_masked_prefill_bf16(const void* q, int ldq, void* o
                                                  int dv, const void* cache, int page_tokens, const int* block_table,
                                                  int max_blocks, const int* positions, const int* row_seg,
                                                  const int* tile_row0, const int* tile_rows, int n_tiles, int mask,
-                                                 int mask_size, int sink, float scale, hipStream_t stream) {
+                                                 int mask_size, int sink, float scale, int key_parts, int out_f32,
+                                                 hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale);
+  int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale, key_parts, out_f32);
   if (e) return e;
   n_tiles *= 2;  // halves
   if (max_blocks <= 0 || (long)n_tiles * H > 0x7fffffffL) return APC_ERR_BAD_ARG;
   dim3 grid(n_tiles * H), block(256);
 #define MP_LAUNCH(DK_, DV_)                                                                                         \
   hipLaunchKernelGGL((attn_masked_prefill_kernel<DK_, DV_>), grid, block, 0, stream, (const bf16_t*)q, ldq,          \
-                     (bf16_t*)out, ldo, H, G, dk, dv, (const bf16_t*)cache, page_tokens, block_table, max_blocks,    \
-                     positions, row_seg, tile_row0, tile_rows, n_tiles, mask, mask_size, sink, scale)
+                     out, ldo, H, G, dk, dv, (const bf16_t*)cache, page_tokens, block_table, max_blocks,             \
+                     positions, row_seg, tile_row0, tile_rows, n_tiles, mask, mask_size, sink, scale, key_parts,    \
+                     out_f32)
 #define MP_VALUES(DK_)                       \
   do {                                       \
     if (dv <= 64) MP_LAUNCH(DK_, 64);        \
@@ -512,11 +528,12 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
                                                 int dk, int dv, const void* cache, int page_tokens,
                                                 const int* block_table, int max_blocks, const int* positions,
                                                 const int* row_seg, const int* rows, int mask, int mask_size, int sink,
-                                                float scale, int n_splits, float* parts, hipStream_t stream) {
+                                                float scale, int n_splits, float* parts, int key_parts, int out_f32,
+                                                hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale);
+  int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale, key_parts, out_f32);
   if (e) return e;
-  if (!apc_attention_masked_takes(H, G, dk, dv, page_tokens)) return APC_ERR_UNSUPPORTED;
+  if (!apc_attention_masked_takes(H, G, dk, dv, page_tokens, key_parts)) return APC_ERR_UNSUPPORTED;
   if (n_splits <= 0 || n_splits > WAVE || !parts || max_blocks <= 0 ||
       (long)n_rows * G * n_splits > 0x7fffffffL || H > 65535)
     return APC_ERR_BAD_ARG;
@@ -524,7 +541,7 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
 #define MD_LAUNCH(KS_, ET_)                                                                                       \
   hipLaunchKernelGGL((attn_masked_decode_kernel<KS_, ET_>), grid, block, 0, stream, (const bf16_t*)q, ldq, H, G, dk, \
                      dv, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg, rows, mask,  \
-                     mask_size, scale, n_splits, parts)
+                     mask_size, scale, n_splits, parts, key_parts)
 #define MD_VALUES(KS_)                     \
   do {                                     \
     if (dv <= 64) MD_LAUNCH(KS_, 4);       \
@@ -538,7 +555,7 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
 #undef MD_LAUNCH
   APC_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn_masked_merge_kernel, dim3(n_rows, H), dim3(64), 0, stream, parts, n_splits, H, dv, rows, sink,
-                     (bf16_t*)out, ldo);
+                     out, ldo, out_f32);
   APC_LAUNCH_CHECK();
   return 0;
 }

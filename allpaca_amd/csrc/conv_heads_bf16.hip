@@ -1,6 +1,8 @@
 // The short convolution on the heads of projected rows (see plain_mixers.hip for the formulas) for bfloat16 rows, 16
 // bytes a thread: a block takes 8 or 4 consecutive rows whole, a thread PPT pieces of 8 channels of each, with the taps of
-// its channels in registers.  Sums of squares of the pieces go through LDS, so a head may be any multiple of 8 wide.
+// its channels in registers.  Sums of squares of the pieces go through LDS, so a head may be any multiple of 8 wide,
+// and so may the width the norm is taken over (`norm_dim`, which divides a head; the normed values are multiplied with
+// q_norm_w / k_norm_w [norm_dim] if given).
 // The row holds q heads, then k heads, then v heads.  The state of the convolution is moved on by the plain kernel,
 // or here (`fold_state`) in a step of few rows in which every segment is a single row (decoded tokens).
 #include "mfma.h"
@@ -23,7 +25,8 @@ __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
     const bf16_t* __restrict__ proj, int ld, int n_rows, int H, int G, int dk, int dv, const float* __restrict__ bias,
     const float* __restrict__ conv_w, float* __restrict__ state, int fold_state, int width,
     const int* __restrict__ row_seg, const int* __restrict__ seg_row0, const int* __restrict__ slots,
-    const int* __restrict__ positions, int unit_norm, float eps, bf16_t* __restrict__ q_out, int ldq,
+    const int* __restrict__ positions, int unit_norm, float eps, int norm_dim, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, bf16_t* __restrict__ q_out, int ldq,
     const int* __restrict__ block_table, int max_blocks, bf16_t* __restrict__ cache, int P) {
   extern __shared__ float ssum[];            // [ROWS][pieces]
   constexpr int taps = TAPS;
@@ -151,20 +154,30 @@ __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
     const int d = kind == 2 ? dv : dk;
     const int rel = c0 - (kind == 0 ? 0 : kind == 1 ? kq : kk);
     const int head = rel / d, off = rel % d;
+    const int noff = off % norm_dim;                 // the piece's place in the range its norm is taken over
+    float nw[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) nw[e] = 1.f;
+    const float* nwp = kind == 0 ? q_norm_w : kind == 1 ? k_norm_w : nullptr;
+    if (nwp) {
+      const float4 a = *reinterpret_cast<const float4*>(nwp + noff), c = *reinterpret_cast<const float4*>(nwp + noff + 4);
+      nw[0] = a.x; nw[1] = a.y; nw[2] = a.z; nw[3] = a.w; nw[4] = c.x; nw[5] = c.y; nw[6] = c.z; nw[7] = c.w;
+    }
 #pragma unroll
     for (int rr = 0; rr < ROWS; ++rr) {
       const int r = r0 + rr;
       if (r >= n_rows) continue;
       float inv = 1.f;
       if (unit_norm && kind != 2) {
-        const float* sp = ssum + rr * pieces + (c0 - off) / 8;
+        const float* sp = ssum + rr * pieces + (c0 - noff) / 8;
         float ss = 0.f;
-        for (int i = 0; i < d / 8; ++i) ss += sp[i];
-        inv = 1.0f / sqrtf(ss / (float)d + eps);
+        for (int i = 0; i < norm_dim / 8; ++i) ss += sp[i];
+        inv = 1.0f / sqrtf(ss / (float)norm_dim + eps);
       }
       Frag o;
 #pragma unroll
-      for (int wd = 0; wd < 4; ++wd) o.w[wd] = pack_bf16x2(y[k][rr][2 * wd] * inv, y[k][rr][2 * wd + 1] * inv);
+      for (int wd = 0; wd < 4; ++wd)
+        o.w[wd] = pack_bf16x2((y[k][rr][2 * wd] * inv) * nw[2 * wd], (y[k][rr][2 * wd + 1] * inv) * nw[2 * wd + 1]);
       if (kind == 0) {
         *reinterpret_cast<Frag*>(q_out + (size_t)r * ldq + c0) = o;
         continue;
@@ -195,7 +208,7 @@ APC_EXPORT int apc_conv_heads_bf16_takes(int ld, int width, int H, int G, int dk
 APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, int G, int dk, int dv, const float* bias,
                                    const float* conv_w, int taps, float* state, int fold_state, int width, const int* row_seg,
                                    const int* seg_row0, const int* slots, const int* positions, int unit_norm, float eps,
-                                   void* q_out, int ldq, const int* block_table, int max_blocks, void* cache,
+                                   int norm_dim, const float* q_norm_w, const float* k_norm_w, void* q_out, int ldq, const int* block_table, int max_blocks, void* cache,
                                    int page_tokens, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (!apc_conv_heads_bf16_takes(ld, width, H, G, dk, dv, taps, ldq)) return APC_ERR_UNSUPPORTED;
@@ -203,6 +216,9 @@ APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, 
       ((uintptr_t)bias & 15u) || ((uintptr_t)conv_w & 15u))
     return APC_ERR_UNSUPPORTED;
   if (taps > 1 && (!conv_w || !state || !slots)) return APC_ERR_BAD_ARG;
+  if (norm_dim <= 0) norm_dim = dk;
+  if (dk % norm_dim) return APC_ERR_BAD_ARG;
+  if (norm_dim % 8 || ((uintptr_t)q_norm_w & 15u) || ((uintptr_t)k_norm_w & 15u)) return APC_ERR_UNSUPPORTED;
   if (!conv_w && taps != 1) return APC_ERR_BAD_ARG;
   if (G > 0 && (!cache || !block_table || page_tokens <= 0 || max_blocks <= 0)) return APC_ERR_BAD_ARG;
   // A row's pieces of 8 channels are spread over up to 768 threads (a block of 1,024 would leave a thread too few
@@ -218,7 +234,7 @@ APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, 
 #define CH_LAUNCH(NT_, PPT_, ROWS_, TAPS_)                                                                          \
   hipLaunchKernelGGL((conv_heads_bf16_kernel<NT_, PPT_, ROWS_, TAPS_>), grid, block, lds, stream,                   \
                      (const bf16_t*)proj, ld, n_rows, H, G, dk, dv, bias, conv_w, state, fold_state, width, row_seg, seg_row0,  \
-                     slots, positions, unit_norm, eps, (bf16_t*)q_out, ldq, block_table, max_blocks, (bf16_t*)cache, \
+                     slots, positions, unit_norm, eps, norm_dim, q_norm_w, k_norm_w, (bf16_t*)q_out, ldq, block_table, max_blocks, (bf16_t*)cache, \
                      page_tokens)
 #define CH_TAPS(NT_, PPT_, ROWS_)                            \
   do {                                                       \

@@ -417,8 +417,8 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
     if (_tuned_ok(proj, q_out) and (cache is None or cache.dtype == torch.bfloat16) and q_off == 0
             and (G == 0 or (k_off == n_heads * key_dim and v_off == (n_heads + G) * key_dim))):
         LT = _lib.load("tuned")
-        if (LT.apc_conv_heads_bf16_takes(ld, width, n_heads, G, key_dim, value_dim, taps, ldq) and nd == key_dim
-                and q_norm_w is None and k_norm_w is None
+        if (LT.apc_conv_heads_bf16_takes(ld, width, n_heads, G, key_dim, value_dim, taps, ldq) and nd % 8 == 0
+                and all(w is None or w.data_ptr() % 16 == 0 for w in (q_norm_w, k_norm_w))
                 and proj.data_ptr() % 16 == 0 and q_out.data_ptr() % 16 == 0
                 and (cache is None or cache.data_ptr() % 16 == 0) and (state is None or state.data_ptr() % 16 == 0)
                 and (conv_w is None or (conv_w.data_ptr() % 16 == 0 and width % 4 == 0))):
@@ -430,7 +430,8 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
                 _f32(conv_w, width * taps, "conv weights"), taps,
                 state.data_ptr() if taps > 1 else 0, 1 if fold else 0, width, _i32(step.row_seg, T, "row_seg"),
                 _i32(step.seg_row0, S, "seg_row0"), _i32(slots, S, "slots") if taps > 1 else 0,
-                _i32(step.positions, T, "positions"), 1 if unit_norm else 0, float(eps), q_out.data_ptr(), ldq,
+                _i32(step.positions, T, "positions"), 1 if unit_norm else 0, float(eps), nd,
+                _f32(q_norm_w, nd, "q norm weight"), _f32(k_norm_w, nd, "k norm weight"), q_out.data_ptr(), ldq,
                 block_table.data_ptr() if G else 0, max_blocks, cache.data_ptr() if G else 0, page_tokens, _stream()),
                 "conv_heads_bf16")
             if taps > 1 and not fold:

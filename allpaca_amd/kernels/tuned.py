@@ -469,13 +469,14 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
     ldq, ldo = _ops._rows(q, "attention q"), _ops._rows(out, "attention out")
     T = q.shape[0]
     L = _lib.load("tuned")
-    if key_parts != 1:
+    f32 = out.dtype == torch.float32
+    if (not scale > 0 or ldq % 8 or ldo % 4 or not _aligned(q, cache) or out.data_ptr() % (16 if f32 else 8)
+            or q.dtype != torch.bfloat16 or cache.dtype != torch.bfloat16
+            or out.dtype not in (torch.bfloat16, torch.float32)
+            or not L.apc_attention_masked_takes(n_heads, n_kv_heads, key_dim, value_dim, page_tokens, key_parts)):
         return False
-    if (not scale > 0 or ldq % 8 or ldo % 4 or not _aligned(q, cache) or out.data_ptr() % 8
-            or q.dtype != torch.bfloat16 or cache.dtype != torch.bfloat16 or out.dtype != torch.bfloat16
-            or not L.apc_attention_masked_takes(n_heads, n_kv_heads, key_dim, value_dim, page_tokens)):
-        return False
-    _ops._need(q.shape[1] == n_heads * key_dim, "attention: q must be [rows, heads * key_dim]")
+    _ops._check_key_parts(n_heads, n_kv_heads, key_dim, key_parts)
+    _ops._need(q.shape[1] == n_heads * (key_dim // key_parts), "attention: q must be [rows, heads * key_dim / key_parts]")
     _ops._need(out.shape == (T, n_heads * value_dim), "attention out must be [rows, heads * value_dim]")
     _ops._split_pages(cache, n_kv_heads, key_dim, value_dim, page_tokens)
     _ops._need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
@@ -487,7 +488,8 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
             q.data_ptr(), ldq, out.data_ptr(), ldo, n_heads, n_kv_heads, key_dim, value_dim, cache.data_ptr(),
             page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
             step.row_seg.data_ptr(), step.tile_row0.data_ptr(), step.tile_rows.data_ptr(), step.n_tiles, code,
-            int(mask_size), 1 if sink else 0, float(scale), stream), "attention_masked_prefill_bf16")
+            int(mask_size), 1 if sink else 0, float(scale), int(key_parts), 1 if f32 else 0, stream),
+            "attention_masked_prefill_bf16")
     if step.n_decode_rows:
         n = step.n_decode_rows
         keys = min(step.max_decode_context, mask_size) if code else step.max_decode_context
@@ -498,8 +500,8 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
             q.data_ptr(), ldq, out.data_ptr(), ldo, n, n_heads, n_kv_heads, key_dim, value_dim, cache.data_ptr(),
             page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
             step.row_seg.data_ptr(), step.decode_rows.data_ptr() if step.decode_rows is not None else 0, code,
-            int(mask_size), 1 if sink else 0, float(scale), splits, parts.data_ptr(), stream),
-            "attention_masked_decode_bf16")
+            int(mask_size), 1 if sink else 0, float(scale), splits, parts.data_ptr(), int(key_parts),
+            1 if f32 else 0, stream), "attention_masked_decode_bf16")
     return True
 
 
@@ -507,9 +509,66 @@ def rmsnorm_add_f32(y, weight, eps, mult, x, copy) -> bool:
     return False
 
 
+LINEAR_CHUNK_MIN_ROWS = 5    # segments of at least this many rows make a step run on the kernel of 64-row chunks
+
+
 def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, state, step, slots, out) -> bool:
-    return False
+    """Linear attention with a decay on the MFMA kernel that walks a segment in chunks of 64 rows.  False (nothing
+    done) for sizes it does not take and for steps whose segments are all short (decoded rows): the caller then runs
+    the kernel that walks row by row."""
+    ld, ldo = _ops._rows(proj, "projected rows"), _ops._rows(out, "linear attention out")
+    L = _lib.load("tuned")
+    if (step.max_rows < LINEAR_CHUNK_MIN_ROWS or proj.dtype != torch.bfloat16 or ldo % 4 or not _aligned(proj, out)
+            or not L.apc_linear_attention_bf16_takes(ld, q_off, k_off, v_off, H, dk, dv)):
+        return False
+    S = step.n_segs
+    _lib.check(L.apc_linear_attention_bf16(
+        proj.data_ptr(), ld, q_off, k_off, v_off, H, dk, dv, 1 if silu else 0, _ops._f32(decay, H, "decay"),
+        state.data_ptr(), S, _ops._i32(step.seg_row0, S, "seg_row0"), _ops._i32(step.seg_rows, S, "seg_rows"),
+        _ops._i32(slots, S, "slots"), out.data_ptr(), ldo, _ops._stream()), "linear_attention_bf16")
+    return True
 
 
-def pack_experts(gate_up, down):
-    return None
+class PackedExperts:
+    """The matrices of a layer's experts in the tiled layout of the MFMA kernels: `data` holds, for every expert, the
+    tiles of its matrices (`per_expert` of them: gate and up, or down alone), each packed like a `PackedWeight`."""
+
+    def __init__(self, data: torch.Tensor, n_experts: int, N: int, K: int):
+        self.data, self.E, self.N, self.K = data, n_experts, N, K
+
+
+ROUTED_WIDE_TILE_MIN = 32    # pairs an expert on average from which a tile holds 64 rows instead of 16
+
+
+def pack_experts(gate_up: torch.Tensor, down: torch.Tensor):
+    """[E, 2 F, D] and [E, D, F] bfloat16 -> (PackedExperts, PackedExperts), or None for sizes the kernels do not take."""
+    from .packing import pack_mfma
+    E, F2, D = gate_up.shape
+    F = F2 // 2
+    if not _lib.load("tuned").apc_routed_bf16_takes(E, F, D):
+        return None
+    gu = torch.stack([torch.stack([pack_mfma(gate_up[e, :F].contiguous()).data,
+                                   pack_mfma(gate_up[e, F:].contiguous()).data]) for e in range(E)]).contiguous()
+    dn = torch.stack([pack_mfma(down[e].contiguous()).data for e in range(E)]).contiguous()
+    return PackedExperts(gu, E, F, D), PackedExperts(dn, E, D, F)
+
+
+def routed_experts_bf16(h, w_gate_up: PackedExperts, w_down: PackedExperts, E: int, F: int, ids, weights, K: int,
+                        y) -> None:
+    """The chosen experts of every row on the MFMA kernels (pairs sorted by expert on the GPU, nothing read back)."""
+    T, D = h.shape
+    _ops._gpu(h, w_gate_up.data, w_down.data, ids, weights, y)
+    _ops._need(h.dtype == torch.bfloat16 and (w_gate_up.E, w_gate_up.N, w_gate_up.K) == (E, F, D)
+               and (w_down.E, w_down.N, w_down.K) == (E, D, F), "routed experts: matrices do not fit the sizes")
+    L = _lib.load("tuned")
+    n_pairs = T * K
+    tile_rows = 64 if n_pairs >= ROUTED_WIDE_TILE_MIN * E else 16
+    max_tiles = L.apc_routed_max_tiles(n_pairs, E, tile_rows)
+    dev = h.device
+    work = torch.empty(2 * n_pairs + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
+    act = torch.empty((n_pairs, F), dtype=torch.bfloat16, device=dev)
+    ys = torch.empty((n_pairs, D), dtype=torch.float32, device=dev)
+    _lib.check(L.apc_routed_experts_bf16(
+        h.data_ptr(), _ops._rows(h, "h"), w_gate_up.data.data_ptr(), w_down.data.data_ptr(), E, F, D,
+        _ops._i32(ids, n_pairs, "ids"), _ops._f32(weights, n_pairs, "weights"), K, T, tile_rows, work.data_ptr(),
+        act.data_ptr(), ys.data_ptr(), y.data_ptr(), _ops._rows(y, "y"), _ops._stream()), "routed_experts_bf16")
