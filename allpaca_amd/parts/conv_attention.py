@@ -97,7 +97,12 @@ class ConvAttention(Mixer):
             if not self.shares_kv:
                 self.k_norm_w = to_device(tensors[n["k"] + n["norm"]], rt, torch.float32)
         # one [width, D] matrix: a single product gives q (, k and v) of a row
-        self.w_in = ops.prepare_matrix(torch.cat([to_device(m, rt, dt) for m in mats], dim=0), rt.dtype)
+        mats = [to_device(m, rt, dt) for m in mats]
+        # (rows of zeros behind a subclass's extra rows, so that a row of the product is a multiple of 16 bytes)
+        self.full_width = self.width + (-(-self.extra_rows // 8) * 8 if self.extra_rows else 0)
+        if self.full_width > self.width + self.extra_rows:
+            mats.append(torch.zeros((self.full_width - self.width - self.extra_rows, self.D), dtype=dt, device=rt.device))
+        self.w_in = ops.prepare_matrix(torch.cat(mats, dim=0), rt.dtype)
         self.w_o = ops.prepare_matrix(to_device(tensors[n["o"]], rt), rt.dtype)
         self.b_in = self.conv_w = None
         if self.bias:
@@ -114,7 +119,7 @@ class ConvAttention(Mixer):
         pages, state = (cache.get("mixer"), cache.get("mixer.state")) if isinstance(cache, dict) else (cache, None)
         h = as_normed(h).tensor()
         T, dev, dt = h.shape[0], h.device, self.rt.dtype
-        full = torch.empty((T, self.width + self.extra_rows), dtype=dt, device=dev)
+        full = torch.empty((T, self.full_width), dtype=dt, device=dev)
         ops.linear(h, self.w_in, full)
         proj = full[:, :self.width] if self.extra_rows else full
         q = torch.empty((T, self.H * self.dk), dtype=dt, device=dev)

@@ -245,3 +245,14 @@ class PlainGulidra:
                 layers_out.append(x.copy())
         mem.pos += len(tokens)
         return rms_norm(x, w["final.norm"], self.eps) @ w["head"].T
+
+
+def greedy(model: PlainGulidra, prompt, n: int) -> List[int]:
+    """The n tokens that follow `prompt` when the largest logit is taken every time (the lowest id wins a tie)."""
+    mem = model.new_memory()
+    logits = model.forward(list(prompt), mem)[-1]
+    out = []
+    for _ in range(n):
+        out.append(int(np.argmax(logits)))
+        logits = model.forward([out[-1]], mem)[-1]
+    return out
