@@ -44,6 +44,16 @@ struct TiledPre {
   float eps;
 };
 
+// Rows in runs that each multiply with a matrix of their own (routed experts: the rows that chose an expert lie side by
+// side): `tiles` holds (matrix, first row, rows) of every row tile, `*n_tiles` of them, and matrix e starts
+// `w_stride` elements behind matrix e - 1.  The grid is (column tiles, most row tiles there can be); a block beyond
+// the tiles that exist leaves at once.  tiles == nullptr: one matrix for all rows.
+struct GroupedRows {
+  const int* tiles;
+  const int* n_tiles;
+  size_t w_stride;
+};
+
 // EVEN_K: K is a multiple of 64, so no load needs a bound check.  BM: rows of the block tile, 64 or 128.
 // DEPTH (even): how many K steps the global loads run ahead of the MFMAs, one register set a step.  2 where two blocks
 // share a compute unit (many rows); 4 for the steps of up to 128 rows, whose blocks have a unit each and stream the
@@ -54,7 +64,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
                                                         const bf16_t* __restrict__ W,
                                                         const bf16_t* __restrict__ W2, int chunks,
                                                         void* __restrict__ C, int ldc, int M, int N, int K,
-                                                        int k_split, TiledPre pre = TiledPre{}) {
+                                                        int k_split, TiledPre pre = TiledPre{},
+                                                        GroupedRows grp = GroupedRows{nullptr, nullptr, 0}) {
   static_assert(!PRE || MODE == G_STORE_BF16 || MODE == G_STORE_F32 || MODE == G_SWIGLU,
                 "a product that reads a normalised row stores its result");
   __shared__ float rstd_s[PRE ? BM : 1];
@@ -72,6 +83,17 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
   if (MODE == G_PARTIAL) {
     mt = blockIdx.y;
     nt = blockIdx.x;
+  } else if (grp.tiles) {
+    const int ti = blockIdx.y;
+    nt = blockIdx.x;
+    mt = 0;
+    if (ti >= *grp.n_tiles || nt >= ceil_div(N, NB)) return;
+    const int e = grp.tiles[3 * ti], p0 = grp.tiles[3 * ti + 1];
+    M = grp.tiles[3 * ti + 2];                       // the tile's rows are all the rows this block knows of
+    A += (size_t)p0 * lda;
+    C = (char*)C + (size_t)p0 * ldc * (MODE == G_STORE_BF16 || MODE == G_SWIGLU ? 2 : 4);
+    W += (size_t)e * grp.w_stride;
+    if (MODE == G_SWIGLU) W2 += (size_t)e * grp.w_stride;
   } else {
     // Order of the blocks: consecutive block ids go to the 8 XCDs in turn, each with an L2 of its own.  XCD x takes
     // the column tiles x, x+8, ..; inside it, groups of up to 8 row tiles sweep those columns, row tile fastest, so
@@ -612,6 +634,41 @@ APC_EXPORT int apc_gemm_bf16(const void* A, int lda, const void* W, void* C, int
     case G_ACC_F32: return launch_gemm<G_ACC_F32>(a, lda, w, nullptr, C, ldc, M, N, K, stream);
     default: return APC_ERR_BAD_ARG;
   }
+}
+
+// Rows in runs of one matrix each (see GroupedRows): mode G_SWIGLU (W, W2: gate and up; bfloat16 out) or G_STORE_F32.
+// tile_rows: 64 or 128, the rows `tiles` was cut for.
+APC_EXPORT int apc_gemm_grouped_bf16(const void* A, int lda, const void* W, const void* W2, size_t w_stride, void* C,
+                                     int ldc, const int* tiles, const int* n_tiles, int max_tiles, int tile_rows,
+                                     int N, int K, int mode, hipStream_t stream) {
+  if (max_tiles <= 0) return 0;
+  if (N <= 0 || K <= 0 || K % 8 || lda % 8 || !tiles || !n_tiles || (tile_rows != 64 && tile_rows != 128) ||
+      (mode != G_SWIGLU && mode != G_STORE_F32) || (mode == G_SWIGLU && !W2) || max_tiles > 65535)
+    return APC_ERR_BAD_ARG;
+  if (!aligned16(A) || !aligned16(W) || (W2 && !aligned16(W2))) return APC_ERR_UNSUPPORTED;
+  const GroupedRows grp{tiles, n_tiles, w_stride};
+  const int nb = mode == G_SWIGLU ? BN / 2 : BN;
+  const dim3 grid(ceil_div(N, nb), max_tiles);
+#define GROUPED_LAUNCH(MODE_, EVEN_, BM_)                                                                          \
+  hipLaunchKernelGGL((gemm_bf16_kernel<MODE_, EVEN_, BM_, false, 2>), grid, dim3(256), 0, stream, (const bf16_t*)A, \
+                     lda, (const bf16_t*)W, (const bf16_t*)W2, ceil_div(K, 32), C, ldc, tile_rows, N, K, 1,        \
+                     TiledPre{}, grp)
+#define GROUPED_BY(MODE_)                                                    \
+  do {                                                                       \
+    if (tile_rows == 64) {                                                   \
+      if (K % BK == 0) GROUPED_LAUNCH(MODE_, true, 64);                      \
+      else GROUPED_LAUNCH(MODE_, false, 64);                                 \
+    } else {                                                                 \
+      if (K % BK == 0) GROUPED_LAUNCH(MODE_, true, BM_ROWS);                 \
+      else GROUPED_LAUNCH(MODE_, false, BM_ROWS);                            \
+    }                                                                        \
+  } while (0)
+  if (mode == G_SWIGLU) GROUPED_BY(G_SWIGLU);
+  else GROUPED_BY(G_STORE_F32);
+#undef GROUPED_BY
+#undef GROUPED_LAUNCH
+  APC_LAUNCH_CHECK();
+  return 0;
 }
 
 APC_EXPORT int apc_gemm_swiglu_bf16(const void* A, int lda, const void* Wg, const void* Wu, void* C, int ldc, int M,

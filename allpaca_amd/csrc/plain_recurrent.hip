@@ -10,6 +10,12 @@ namespace {
 
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 
+// silu of a projected value, held in the rows' own element type like every activation of a run
+__device__ __forceinline__ float act_silu(float z, int dtype) {
+  const float a = z * sigmoid_f(z);
+  return dtype == APC_BF16 ? bf16_to_float(float_to_bf16(a)) : a;
+}
+
 // x[t] = table[tokens[t]] * scale + pos_table[positions[t]]
 __global__ void embed_positions_kernel(const void* __restrict__ table, int table_dtype, const int* __restrict__ tokens,
                                        const void* __restrict__ pos_table, int pos_dtype,
@@ -42,6 +48,58 @@ __global__ __launch_bounds__(NT) void rmsnorm_add_kernel(const void* __restrict_
     const float nx = x[(size_t)r * ldx + i] + mult * ((v * inv) * w[i]);
     x[(size_t)r * ldx + i] = nx;
     if (copy) store_f(copy, copy_dtype, (size_t)r * ldc + i, nx);
+  }
+}
+
+// The same for float32 rows whose width is a multiple of 4 and at most NT*4*VPT: every thread keeps its elements of
+// y in registers between the sum and the scaling, and all its loads are in flight together.  Which of the two kernels
+// runs, and so the order of the additions, is fixed by the width and the alignment of the rows alone.
+template <int NT, int VPT>
+__global__ __launch_bounds__(NT) void rmsnorm_add_f4_kernel(const float* __restrict__ y, int ldy,
+                                                            const float* __restrict__ w, float eps, float mult,
+                                                            float* __restrict__ x, int ldx, void* __restrict__ copy,
+                                                            int copy_dtype, int ldc, int dim) {
+  __shared__ float red[NT / WAVE];
+  const int r = blockIdx.x, n4 = dim / 4;
+  const float4* src = reinterpret_cast<const float4*>(y + (size_t)r * ldy);
+  float4* xr = reinterpret_cast<float4*>(x + (size_t)r * ldx);
+  float4 v[VPT], old[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * NT;
+    v[j] = i < n4 ? src[i] : float4{0.f, 0.f, 0.f, 0.f};
+    old[j] = i < n4 ? xr[i] : float4{0.f, 0.f, 0.f, 0.f};
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    ss = fmaf(v[j].x, v[j].x, ss);
+    ss = fmaf(v[j].y, v[j].y, ss);
+    ss = fmaf(v[j].z, v[j].z, ss);
+    ss = fmaf(v[j].w, v[j].w, ss);
+  }
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+  const float4* w4 = reinterpret_cast<const float4*>(w);
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * NT;
+    if (i >= n4) continue;
+    const float4 g = w4[i];
+    const float4 nx = float4{old[j].x + mult * ((v[j].x * inv) * g.x), old[j].y + mult * ((v[j].y * inv) * g.y),
+                             old[j].z + mult * ((v[j].z * inv) * g.z), old[j].w + mult * ((v[j].w * inv) * g.w)};
+    xr[i] = nx;
+    if (copy) {
+      const size_t at = (size_t)r * ldc + (size_t)i * 4;
+      if (copy_dtype == APC_F32) {
+        *reinterpret_cast<float4*>((float*)copy + at) = nx;
+      } else {
+        uint2 pk;
+        pk.x = pack_bf16x2(nx.x, nx.y);
+        pk.y = pack_bf16x2(nx.z, nx.w);
+        *reinterpret_cast<uint2*>((bf16_t*)copy + at) = pk;
+      }
+    }
   }
 }
 
@@ -78,12 +136,12 @@ __global__ __launch_bounds__(256) void linear_attention_kernel(
     for (int i = tid; i < dk; i += 256) {
       float qv = load_f(proj, in_dtype, row + q_off + (size_t)h * dk + i);
       float kv = load_f(proj, in_dtype, row + k_off + (size_t)h * dk + i);
-      if (act) { qv = qv * sigmoid_f(qv); kv = kv * sigmoid_f(kv); }
+      if (act) { qv = act_silu(qv, in_dtype); kv = act_silu(kv, in_dtype); }
       qs[b][i] = qv;
       ks[b][i] = kv;
     }
     float vv = on ? load_f(proj, in_dtype, row + v_off + (size_t)h * dv + col) : 0.f;
-    if (act) vv = vv * sigmoid_f(vv);
+    if (act) vv = act_silu(vv, in_dtype);
     __syncthreads();
     float acc = 0.f;
 #pragma unroll
@@ -172,8 +230,23 @@ APC_EXPORT int apc_rmsnorm_add(const void* y, int y_dtype, int ldy, const float*
                                int ldx, void* copy, int copy_dtype, int ldc, int n_rows, int dim, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (dim <= 0 || ldy < dim || ldx < dim || (copy && ldc < dim)) return APC_ERR_BAD_ARG;
-  hipLaunchKernelGGL(rmsnorm_add_kernel<256>, dim3(n_rows), dim3(256), 0, stream, y, y_dtype, ldy, w, eps, mult, x, ldx,
-                     copy, copy_dtype, ldc, dim);
+  const bool vec = y_dtype == APC_F32 && dim % 4 == 0 && ldy % 4 == 0 && ldx % 4 == 0 && (!copy || ldc % 4 == 0) &&
+                   dim <= 256 * 4 * 8 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)x % 16) == 0 &&
+                   ((uintptr_t)w % 16) == 0 && ((uintptr_t)copy % 16) == 0;
+  if (vec) {
+    const int n4 = dim / 4;
+#define RA_LAUNCH(VPT_)                                                                                          \
+  hipLaunchKernelGGL((rmsnorm_add_f4_kernel<256, VPT_>), dim3(n_rows), dim3(256), 0, stream, (const float*)y, ldy, \
+                     w, eps, mult, x, ldx, copy, copy_dtype, ldc, dim)
+    if (n4 <= 256) RA_LAUNCH(1);
+    else if (n4 <= 512) RA_LAUNCH(2);
+    else if (n4 <= 1024) RA_LAUNCH(4);
+    else RA_LAUNCH(8);
+#undef RA_LAUNCH
+  } else {
+    hipLaunchKernelGGL(rmsnorm_add_kernel<256>, dim3(n_rows), dim3(256), 0, stream, y, y_dtype, ldy, w, eps, mult, x,
+                       ldx, copy, copy_dtype, ldc, dim);
+  }
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -4,6 +4,10 @@
 //             (`order`: sorted place -> pair, `place`: pair -> sorted place), and every expert's run is cut into tiles
 //             of `tile_rows` rows (`tiles`: expert, first place, rows).  The order inside a run is whatever the
 //             atomics give; no result depends on it, since every pair's output is computed for itself.
+//   With many rows an expert (tiles of 64 or 128 rows) the rows are copied side by side first (`gather`) and the two
+//   products run on the tiled kernel of the other products in its grouped mode (gemm_bf16.hip): the same tiles through
+//   LDS, the matrix chosen per row tile.  With few (tiles of 16 rows: decoded rows) they run on the kernels below,
+//   which stream an expert's matrices once a tile straight into the MFMA operands:
 //   gate/up   a block takes a tile x 4 bands of 16 outputs, a wave one band of the gate matrix and the same band of the
 //             up matrix: the weights' tiles (1 KiB each, in the lane order of the MFMA operand) stream from memory once
 //             a tile, the rows are gathered through `order`; silu(g) * u leaves in bfloat16 at the sorted place.
@@ -169,6 +173,22 @@ __global__ __launch_bounds__(256) void routed_down_bf16_kernel(const bf16_t* __r
   }
 }
 
+// rows side by side in the sorted order: hs[place] = h[row of the pair at that place], 16 bytes a thread
+__global__ __launch_bounds__(256) void routed_gather_kernel(const bf16_t* __restrict__ h, int ldh, int D,
+                                                            const int* __restrict__ order, int K,
+                                                            const int* __restrict__ tiles,
+                                                            const int* __restrict__ n_tiles, int tile_rows,
+                                                            bf16_t* __restrict__ hs) {
+  const int ti = blockIdx.x;
+  if (ti >= *n_tiles) return;
+  const int p0 = tiles[3 * ti + 1], rows = tiles[3 * ti + 2];
+  const int pieces = D / 8;
+  for (int idx = threadIdx.x; idx < rows * pieces; idx += 256) {
+    const int r = idx / pieces, c = (idx % pieces) * 8;
+    *reinterpret_cast<Frag*>(hs + (size_t)(p0 + r) * D + c) = load_frag(h + (size_t)(order[p0 + r] / K) * ldh + c);
+  }
+}
+
 __global__ __launch_bounds__(256) void routed_combine_kernel(const float* __restrict__ ys, const int* __restrict__ place,
                                                              const float* __restrict__ weights, int K,
                                                              const bf16_t* __restrict__ h, int ldh,
@@ -197,14 +217,20 @@ APC_EXPORT int apc_routed_max_tiles(int n_pairs, int E, int tile_rows) {
   return (n_pairs + tile_rows - 1) / tile_rows + (E < n_pairs ? E : n_pairs);
 }
 
+extern "C" int apc_gemm_grouped_bf16(const void* A, int lda, const void* W, const void* W2, size_t w_stride, void* C,
+                                     int ldc, const int* tiles, const int* n_tiles, int max_tiles, int tile_rows,
+                                     int N, int K, int mode, hipStream_t stream);
+
 // work: int32 [2 * n_pairs + 3 * max_tiles + 1] (order, place, tiles, the tiles' count); act: bfloat16 [n_pairs, F];
-// ys: float32 [n_pairs, D].  tile_rows: 16 or 64.
+// ys: float32 [n_pairs, D]; hs: bfloat16 [n_pairs, D] (tiles of 64 and 128 rows only).  tile_rows: 16, 64 or 128.
 APC_EXPORT int apc_routed_experts_bf16(const void* h, int ldh, const void* w_gate_up, const void* w_down, int E, int F,
                                        int D, const int* ids, const float* weights, int K, int n_rows, int tile_rows,
-                                       int* work, void* act, float* ys, float* y, int ldy, hipStream_t stream) {
+                                       int* work, void* act, float* ys, void* hs, float* y, int ldy,
+                                       hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (!apc_routed_bf16_takes(E, F, D)) return APC_ERR_UNSUPPORTED;
-  if (K <= 0 || ldh < D || ldy < D || ldh % 8 || (tile_rows != 16 && tile_rows != 64) || !work || !act || !ys ||
+  if (K <= 0 || ldh < D || ldy < D || ldh % 8 || (tile_rows != 16 && tile_rows != 64 && tile_rows != 128) || !work ||
+      !act || !ys || (tile_rows != 16 && (!hs || ((uintptr_t)hs & 15u))) ||
       ((uintptr_t)h & 15u) || ((uintptr_t)w_gate_up & 15u) || ((uintptr_t)w_down & 15u) || ((uintptr_t)act & 15u) ||
       ((uintptr_t)ys & 15u) || (long)n_rows * K > 0x3fffffffL)
     return APC_ERR_BAD_ARG;
@@ -225,14 +251,21 @@ APC_EXPORT int apc_routed_experts_bf16(const void* h, int ldh, const void* w_gat
     APC_LAUNCH_CHECK();
     hipLaunchKernelGGL(routed_down_bf16_kernel<1>, g2, dim3(256), 0, stream, (const bf16_t*)act, F, D,
                        (const bf16_t*)w_down, tiles, n_tiles, ys);
-  } else {
-    hipLaunchKernelGGL(routed_glu_bf16_kernel<4>, g1, dim3(256), 0, stream, (const bf16_t*)h, ldh,
-                       (const bf16_t*)w_gate_up, F, D, order, K, tiles, n_tiles, (bf16_t*)act);
     APC_LAUNCH_CHECK();
-    hipLaunchKernelGGL(routed_down_bf16_kernel<4>, g2, dim3(256), 0, stream, (const bf16_t*)act, F, D,
-                       (const bf16_t*)w_down, tiles, n_tiles, ys);
+  } else {
+    if (max_tiles > 65535) return APC_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(routed_gather_kernel, dim3(max_tiles), dim3(256), 0, stream, (const bf16_t*)h, ldh, D, order, K,
+                       tiles, n_tiles, tile_rows, (bf16_t*)hs);
+    APC_LAUNCH_CHECK();
+    const size_t gate_elems = (size_t)ceil_div(F, 16) * ceil_div(D, 32) * TILE_ELEMS;
+    const size_t down_elems = (size_t)ceil_div(D, 16) * ceil_div(F, 32) * TILE_ELEMS;
+    int e = apc_gemm_grouped_bf16(hs, D, w_gate_up, (const bf16_t*)w_gate_up + gate_elems, 2 * gate_elems, act, F,
+                                  tiles, n_tiles, max_tiles, tile_rows, F, D, /* SwiGLU */ 3, stream);
+    if (e) return e;
+    e = apc_gemm_grouped_bf16(act, F, w_down, nullptr, down_elems, ys, D, tiles, n_tiles, max_tiles, tile_rows, D, F,
+                              /* float32 out */ 1, stream);
+    if (e) return e;
   }
-  APC_LAUNCH_CHECK();
   hipLaunchKernelGGL(routed_combine_kernel, dim3(n_rows), dim3(256), 0, stream, ys, place, weights, K,
                      (const bf16_t*)h, ldh, y, ldy, D);
   APC_LAUNCH_CHECK();

@@ -587,18 +587,13 @@ def embed_positions(table: torch.Tensor, tokens: torch.Tensor, pos_table: torch.
 
 
 def rmsnorm_add(y: torch.Tensor, weight: torch.Tensor, eps: float, mult: float, x: torch.Tensor,
-                copy: Optional[torch.Tensor] = None, narrow_run: bool = False) -> None:
-    """x += mult * rms_norm(y) * weight, in 32-bit; `copy` (if given) receives the new x in its own element type.
-    `narrow_run`: the step belongs to a bfloat16 run (its kernel library may take the launch)."""
+                copy: Optional[torch.Tensor] = None) -> None:
+    """x += mult * rms_norm(y) * weight, in 32-bit; `copy` (if given) receives the new x in its own element type."""
     _gpu(y, weight, x, copy)
     ldy, ldx = _rows(y, "rmsnorm_add y"), _rows(x, "rmsnorm_add x")
     T, D = x.shape
     _need(x.dtype == torch.float32 and y.shape == (T, D), "rmsnorm_add: x float32 [rows, width], y of the same shape")
     _need(copy is None or copy.shape == (T, D), "rmsnorm_add: the copy must have x's shape")
-    if narrow_run and not FORCE_PLAIN and y.dtype == torch.float32 and (copy is None or copy.dtype == torch.bfloat16):
-        from . import tuned
-        if tuned.rmsnorm_add_f32(y, weight, eps, mult, x, copy):
-            return
     L = _lib.load("plain")
     _lib.check(L.apc_rmsnorm_add(y.data_ptr(), _code(y), ldy, _f32(weight, D, "norm weight"), float(eps), float(mult),
                                  x.data_ptr(), ldx, copy.data_ptr() if copy is not None else 0,

@@ -505,10 +505,6 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
     return True
 
 
-def rmsnorm_add_f32(y, weight, eps, mult, x, copy) -> bool:
-    return False
-
-
 LINEAR_CHUNK_MIN_ROWS = 5    # segments of at least this many rows make a step run on the kernel of 64-row chunks
 
 
@@ -537,7 +533,9 @@ class PackedExperts:
         self.data, self.E, self.N, self.K = data, n_experts, N, K
 
 
-ROUTED_WIDE_TILE_MIN = 32    # pairs an expert on average from which a tile holds 64 rows instead of 16
+# pairs an expert on average from which a row tile holds 64 and 128 rows instead of 16 (and the products run on the
+# tiled kernel through LDS instead of streaming an expert's matrices once a tile)
+ROUTED_TILE_64_MIN, ROUTED_TILE_128_MIN = 24, 96
 
 
 def pack_experts(gate_up: torch.Tensor, down: torch.Tensor):
@@ -562,13 +560,15 @@ def routed_experts_bf16(h, w_gate_up: PackedExperts, w_down: PackedExperts, E: i
                and (w_down.E, w_down.N, w_down.K) == (E, D, F), "routed experts: matrices do not fit the sizes")
     L = _lib.load("tuned")
     n_pairs = T * K
-    tile_rows = 64 if n_pairs >= ROUTED_WIDE_TILE_MIN * E else 16
+    tile_rows = 128 if n_pairs >= ROUTED_TILE_128_MIN * E else 64 if n_pairs >= ROUTED_TILE_64_MIN * E else 16
     max_tiles = L.apc_routed_max_tiles(n_pairs, E, tile_rows)
     dev = h.device
     work = torch.empty(2 * n_pairs + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
     act = torch.empty((n_pairs, F), dtype=torch.bfloat16, device=dev)
     ys = torch.empty((n_pairs, D), dtype=torch.float32, device=dev)
+    hs = torch.empty((n_pairs, D), dtype=torch.bfloat16, device=dev) if tile_rows != 16 else None
     _lib.check(L.apc_routed_experts_bf16(
         h.data_ptr(), _ops._rows(h, "h"), w_gate_up.data.data_ptr(), w_down.data.data_ptr(), E, F, D,
         _ops._i32(ids, n_pairs, "ids"), _ops._f32(weights, n_pairs, "weights"), K, T, tile_rows, work.data_ptr(),
-        act.data_ptr(), ys.data_ptr(), y.data_ptr(), _ops._rows(y, "y"), _ops._stream()), "routed_experts_bf16")
+        act.data_ptr(), ys.data_ptr(), hs.data_ptr() if hs is not None else 0, y.data_ptr(), _ops._rows(y, "y"),
+        _ops._stream()), "routed_experts_bf16")

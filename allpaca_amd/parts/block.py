@@ -227,10 +227,10 @@ class SublayerNorm:
         last = ffn is None
         wants = isinstance(next_norm, ReadsResidual)
         h = copy() if (not last or wants) else None
-        ops.rmsnorm_add(y, w, eps, mult, x, h, narrow_run=narrow)
+        ops.rmsnorm_add(y, w, eps, mult, x, h)
         if not last:
             y = ffn.forward(h if narrow else x, step)
             w, eps = parts["ffn_norm"].rms_params()
             h = copy() if wants else None
-            ops.rmsnorm_add(y, w, eps, mult, x, h, narrow_run=narrow)
+            ops.rmsnorm_add(y, w, eps, mult, x, h)
         return RowsLeft(h) if (wants and narrow) else None

@@ -459,6 +459,117 @@ def design_configs(size: str, layers: int, chunk: int, streams: int = 2, taps: i
     return {"risizen": risizen, "llama": llama}
 
 
+# ---- the Gulidra design beside the llama decoder at equal sizes ---------------------------------------------------
+GULIDRA_LIKE_KERNELS = {
+    "apc_conv_heads_bf16": ["apc_rope_kv_write_bf16", "apc_rope_kv_write"],
+    "apc_attention_masked_prefill_bf16": ["apc_attention_prefill_bf16"],
+    "apc_attention_masked_decode_bf16": ["apc_attention_decode_bf16"],
+    "apc_linear_attention_bf16": ["apc_attention_prefill_bf16"],
+    "apc_linear_attention": ["apc_attention_decode_bf16"],
+    "apc_routed_experts_bf16": ["apc_gemm_swiglu_bf16", "apc_skinny_swiglu_bf16", "apc_skinny_swiglu_pre_bf16"],
+    "apc_rmsnorm_add": ["apc_rmsnorm_rows"],
+    "apc_embed_positions": ["apc_embed_rows", "apc_embed_rows_tiled"],
+    "apc_diff_combine": [],
+    "apc_gated_rmsnorm": [],
+    "apc_route_topk": [],
+}
+GULIDRA_EXPERTS, GULIDRA_IDENTITY, GULIDRA_TOP = 8, 1, 2
+
+
+def gulidra_configs(size: str, context: int, taps: int = 4):
+    """Four layers at the widths of `size`: differential attention (two maps of half a head each, values of a whole
+    head) with a dense feed-forward, linear attention with routed experts (2 of 8 + 1, each half as wide as the dense
+    feed-forward: the same arithmetic a row), an attention that borrows the first one's keys with routed experts, and
+    an attention of its own with a dense feed-forward; the llama decoder with four layers of the same widths."""
+    D, H, G, d, F, V = DESIGN_SIZES[size]
+    att = dict(heads=H, kv_heads=G, dim=d // 2, vdim=d, scale=(d // 2) ** -0.5, diff=0.3, conv=taps)
+    lin = dict(heads=H, dim=d, vdim=d, decay=[1.0 - 2.0 ** -(5 + 3 * i / max(1, H - 1)) for i in range(H)])
+    moe = dict(kind="moe", expert=dict(ff=F // GULIDRA_TOP),
+               router=dict(experts=GULIDRA_EXPERTS, identity=GULIDRA_IDENTITY, top=GULIDRA_TOP))
+    dense = dict(kind="dense", ff=F)
+    gulidra = dict(architecture="Gulidra", vocab=V, width=D, max_positions=2 * context + 4096, embedding=dict(scale=1.0),
+                   residual_mult=0.5, norm=dict(eps=1e-6),
+                   layers=[dict(type="attention", mixer=dict(att), mlp=dense),
+                           dict(type="lightning", mixer=lin, mlp=moe),
+                           dict(type="attention", mixer=dict(att, kv_from=0), mlp=moe),
+                           dict(type="attention", mixer=dict(att), mlp=dense)])
+    return {"gulidra": gulidra, "llama": design_configs(size, 4, 2 * context)["llama"]}
+
+
+def gulidra_rooflines(size, batch, context, T, points):
+    """For the kernels the design adds and their like kernels of the llama decoder: the bytes or the arithmetic of the
+    launches of a step over the measured time, as a share of the GPU's peak (8 TB/s, 2.5 PFLOP/s)."""
+    D, H, G, d, F, V = DESIGN_SIZES[size]
+    Fe, E, K = F // GULIDRA_TOP, GULIDRA_EXPERTS, GULIDRA_TOP
+
+    def work(name, model, rows, keys_sum):
+        """(bytes, flops) of all of a step's launches of entry point `name` in `model`."""
+        att_own, att_all, lin, moe, layers = (2, 3, 1, 2, 4) if model == "gulidra" else (4, 4, 0, 0, 4)
+        if name == "apc_conv_heads_bf16":        # rows read, q and the pages' rows written (a borrower: q alone)
+            own, q = (H + 2 * G) * d, H * d
+            return rows * (att_own * (own + q + 2 * G * d) + (att_all - att_own) * 2 * q) * 2, 0
+        if name in ("apc_rope_kv_write_bf16", "apc_rope_kv_write"):
+            return layers * rows * ((H + 2 * G) * d + H * d + 2 * G * d) * 2, 0
+        if name in ("apc_attention_masked_prefill_bf16", "apc_attention_prefill_bf16"):
+            return 0, att_all * 4 * keys_sum * H * d
+        if name in ("apc_attention_masked_decode_bf16", "apc_attention_decode_bf16"):
+            return att_all * keys_sum * G * 2 * d * 2, 0
+        if name == "apc_linear_attention_bf16":      # scores and their use inside chunks of 64, state read and moved on
+            return 0, lin * rows * H * (2 * 64 * d + 2 * 64 * d + 4 * d * d) // 2 * 2
+        if name == "apc_linear_attention":           # the state of every row read and written
+            return lin * rows * H * d * d * 4 * 2, 0
+        if name == "apc_routed_experts_bf16":
+            used = min(E, rows * K)
+            return moe * used * 3 * Fe * D * 2, moe * rows * K * 3 * 2 * Fe * D
+        if name in ("apc_gemm_swiglu_bf16", "apc_skinny_swiglu_bf16", "apc_skinny_swiglu_pre_bf16"):
+            return layers * 2 * F * D * 2, layers * rows * 2 * 2 * F * D
+        if name == "apc_rmsnorm_add":                # y and x read, x and its copy written
+            return (2 * layers) * rows * D * (4 + 4 + 4 + 2), 0
+        if name == "apc_rmsnorm_rows":
+            return (2 * layers + 1) * rows * D * (4 + 2), 0
+        return None
+
+    table = {}
+    for phase, rows, keys_sum in (("prefill", T, T * (T + 1) // 2), ("decode", batch, batch * context)):
+        for new, likes in GULIDRA_LIKE_KERNELS.items():
+            row = {}
+            for model, names in (("gulidra", [new]), ("llama", likes)):
+                us = sum(points[model][phase + "_kernels_us"].get(n, 0.0) for n in names)
+                name = next((n for n in names if n in points[model][phase + "_kernels_us"]), None)
+                if not us or name is None:
+                    continue
+                w = work(name, model, rows, keys_sum)
+                row[model] = {"us": round(us, 1)}
+                if w:
+                    row[model]["share_of_peak"] = round(max(w[0] / (us * 1e-6) / (HBM_PEAK_GBS * 1e9),
+                                                            w[1] / (us * 1e-6) / PEAK_FLOPS["bf16"]), 4)
+            if row:
+                table[f"{phase}: {new}"] = row
+    return table
+
+
+def gulidra_run(args) -> int:
+    T, batch, context = 2048, args.batch, args.context
+    out = {"metric": "Gulidra beside the llama decoder at equal sizes: prefill tok/s (one prompt of 2048 tokens) and "
+                     f"decode tok/s (batch {batch}, context {context})", "unit": "tok/s", "n_gpus": 1,
+           "dtype": args.dtype, "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
+           "config": {"layers": "attention + dense, linear attention + experts, borrowing attention + experts, "
+                                "attention + dense", "experts": GULIDRA_EXPERTS, "identity": GULIDRA_IDENTITY,
+                      "top": GULIDRA_TOP, "conv_taps": 4, "page_tokens": 16},
+           "sizes": {}}
+    for size in args.design_sizes.split(","):
+        cfgs = gulidra_configs(size, context)
+        points = {m: design_point(c, args.dtype, batch, context, args.steps, args.warmup, T) for m, c in cfgs.items()}
+        out["sizes"][size] = {
+            "shape": dict(zip(("width", "heads", "kv_heads", "head_size", "ff", "vocab"), DESIGN_SIZES[size])),
+            **points,
+            "prefill_gulidra_over_llama": round(points["gulidra"]["prefill_tok_s"] / points["llama"]["prefill_tok_s"], 3),
+            "decode_gulidra_over_llama": round(points["gulidra"]["decode_tok_s"] / points["llama"]["decode_tok_s"], 3),
+            "like_kernels": gulidra_rooflines(size, batch, context, T, points)}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def design_point(cfg_json, dtype, batch, context, steps, warmup, T):
     """Prefill tok/s (one prompt of T tokens in one step), decode tok/s (batch x context, graphs) and the time of
     every kernel in an eager prefill step and an eager decode step of one model."""
@@ -624,7 +735,7 @@ def main() -> int:
                     help="for profiling: only the decode steps at --batch (as --no-points), only the 2,048-token "
                          "prefill (prints its figures as the line's value), or only the sampler over the preset's "
                          "vocabulary (microseconds a step's rows take on the GPU and on the host)")
-    ap.add_argument("--design", choices=["risizen"], default=None,
+    ap.add_argument("--design", choices=["risizen", "gulidra"], default=None,
                     help="instead of the default workload: the named design beside the llama decoder at equal sizes "
                          "(--design-sizes), prefill and decode throughput and the times of their like kernels")
     ap.add_argument("--design-sizes", default="1b,8b", help="with --design: sizes of the comparison, of " + ",".join(DESIGN_SIZES))
@@ -643,6 +754,8 @@ def main() -> int:
     klib.load("plain")
     klib.load("tuned")
 
+    if args.design == "gulidra":
+        return gulidra_run(args)
     if args.design:
         return design_run(args)
     if args.kernel_times:

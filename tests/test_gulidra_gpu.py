@@ -64,7 +64,7 @@ def test_normed_residual_sum(D):
     for narrow in (False, True):
         x = dev(x0)
         copy = torch.empty((5, D), dtype=torch.bfloat16, device=DEV) if narrow else None
-        ops.rmsnorm_add(dev(y), dev(w), 1e-5, 0.6, x, copy, narrow_run=narrow)
+        ops.rmsnorm_add(dev(y), dev(w), 1e-5, 0.6, x, copy)
         want = np.float32(x0) + 0.6 * P.rms_norm(np.float32(y).astype(np.float64), np.float32(w), 1e-5)
         close(x.cpu(), want, "float32", "sum")
         if narrow:
@@ -75,7 +75,7 @@ def _linear_attention_case(rng, H, dk, dv, segs, sharp_at=None):
     T = sum(n for _, n in segs)
     q, k, v = (bf(rng.normal(size=(T, H * d))) for d in (dk, dk, dv))
     if sharp_at is not None:           # one early key and one late query far larger than the rest
-        k[sharp_at] *= 6.0
+        k[sharp_at] *= 8.0             # (powers of two: the values stay ones that bfloat16 holds)
         q[-1] *= 4.0
     return q, k, v
 
@@ -167,6 +167,10 @@ def test_two_maps_a_head_over_pages_with_one_key_that_stands_out(H, G, dq, dv, P
         perm = perm[n:]
     keys = [bf(rng.normal(size=(L, G, 2, dq))) * 0.5 for L in lens]
     vals = [bf(rng.normal(size=(L, G, dv))) for L in lens]
+    targets = (1, (200 // P_) * P_ - 1, (200 // P_) * P_, 269, 270)
+    for t_ in targets[:4]:             # the keys that will be asked for, four times as long as the others
+        keys[0][t_, 0, 0] *= 4.0
+        keys[1][t_, 0, 0] *= 4.0
     pages = np.full((n_pages + 1, G, P_ * (dk + dv)), np.nan, dtype=np.float32)     # what no request wrote is NaN
     for tb, k_, v_ in zip(tables, keys, vals):
         for pos in range(k_.shape[0]):
@@ -176,13 +180,11 @@ def test_two_maps_a_head_over_pages_with_one_key_that_stands_out(H, G, dq, dv, P
     cache = dev(pages, tdt)
     step = make_step(segs, tables, [0, 1, 2])
     T = 72
-    for target in (1, (200 // P_) * P_ - 1, (200 // P_) * P_, 269, 270):
+    for target in targets:
         q = bf(rng.normal(size=(T, H, 2, dq))) * 0.5
         if target < 270:
-            u = keys[0][target, 0, 0] / np.linalg.norm(keys[0][target, 0, 0])
-            q[69, 0, 0] = bf(u * 40.0)
-            u = keys[1][min(target, 300), 0, 0] / np.linalg.norm(keys[1][min(target, 300), 0, 0])
-            q[70, 0, 0] = bf(u * 40.0)
+            q[69, 0, 0] = bf(keys[0][target, 0, 0] / np.linalg.norm(keys[0][target, 0, 0]) * 8.0)
+            q[70, 0, 0] = bf(keys[1][target, 0, 0] / np.linalg.norm(keys[1][target, 0, 0]) * 8.0)
         out = torch.empty((T, H * 2 * dv), dtype=torch.float32, device=DEV)
         ops.masked_attention(dev(q.reshape(T, -1), tdt), out, 2 * H, G, dk, dv, cache, P_, step.block_tables[0], step,
                              "causal", 0, False, 0.8, key_parts=2)
@@ -198,6 +200,8 @@ def test_two_maps_a_head_over_pages_with_one_key_that_stands_out(H, G, dq, dv, P
         if target < 270:
             # the planted key carries the row, almost alone
             w = P.softmax_attention(q[69:70, 0, 0], keys[0][:270, 0, 0], np.eye(270), 0.8)[0]
+            assert w[target] > 0.5, (target, w[target])
+            w = P.softmax_attention(q[70:71, 0, 0], keys[1][:301, 0, 0], np.eye(301), 0.8)[0]
             assert w[target] > 0.5, (target, w[target])
 
 
