@@ -3,8 +3,9 @@
 //   A[t][s] = (q_t . k_s) lam^(t-s) for s <= t                      (scores and decay in float32)
 //   o_t     = lam^(t+1) S0^T q_t + sum_s A[t][s] v_s
 //   S       = lam^n S0 + sum_s (lam^(n-1-s) k_s) v_s^T
-// A block takes one segment x one head x 64 value columns and walks the chunks in order; the state's tile stays in
-// the accumulators of the last product (float32) from chunk to chunk.  q, k and v are bfloat16 (through silu if asked,
+// The chunks of all segments run side by side in three launches: every chunk's own contribution to the state (a block
+// a chunk x head x 64 value columns), then every state element's walk over its segment's chunks, which leaves the
+// state in front of each chunk, then every chunk's outputs.  q, k and v are bfloat16 (through silu if asked,
 // rounded once); everything that is float32 in the formulas and has to be an MFMA operand (S0, the decayed keys, A)
 // goes in as two bfloat16 pieces, value = hi + lo, so that a product keeps 16 bits of it and not 8.
 // All products are transposed (keys or value columns as the rows of a tile) so that a lane holds 4 consecutive
@@ -41,30 +42,37 @@ __device__ __forceinline__ void store_split4(bf16_t* ph, bf16_t* pl, float a, fl
   *reinterpret_cast<uint2*>(pl) = lo;
 }
 
-template <int DKP>  // key size rounded up to a multiple of 64
+// MODE 1: the chunk's own contribution to the state, sum_s (lam^(n-1-s) k_s) v_s^T, into `ws` [chunk][head][dk][dv].
+// MODE 2: the chunk's outputs from the state in front of it, which the scan kernel below has put into `ws` in the
+// contribution's place.  `chunks` [n][2]: a chunk's segment and its first row inside the segment.
+template <int DKP, int MODE>  // key size rounded up to a multiple of 64
 __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
     const bf16_t* __restrict__ proj, int ld, int q_off, int k_off, int v_off, int H, int dk, int dv, int act,
-    const float* __restrict__ decay, float* __restrict__ state, const int* __restrict__ seg_row0,
-    const int* __restrict__ seg_rows, const int* __restrict__ slots, float* __restrict__ out, int ldo) {
+    const float* __restrict__ decay, const int* __restrict__ chunks, float* __restrict__ ws,
+    const int* __restrict__ seg_row0, const int* __restrict__ seg_rows, float* __restrict__ out, int ldo) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   constexpr int QR = DKP + PAD;
   constexpr int IT = DKP / 64;               // tiles of 16 state rows a wave owns
-  bf16_t* Qs = reinterpret_cast<bf16_t*>(lds);   // [C][QR]   q of the chunk's rows
-  bf16_t* Ks = Qs + C * QR;                      // [C][QR]   k
-  bf16_t* Vt = Ks + C * QR;                      // [VT][SR]  v, a column's rows side by side
+  bf16_t* Vt = reinterpret_cast<bf16_t*>(lds);   // [VT][SR]  v, a column's rows side by side
+  // MODE 1
   bf16_t* KtH = Vt + VT * SR;                    // [DKP][SR] decayed k, a key element's rows side by side (hi, lo)
   bf16_t* KtL = KtH + DKP * SR;
-  bf16_t* AsH = KtL + DKP * SR;                  // [C][SR]   A[t][s] (hi, lo)
+  // MODE 2
+  bf16_t* Qs = Vt + VT * SR;                     // [C][QR]   q of the chunk's rows
+  bf16_t* Ks = Qs + C * QR;                      // [C][QR]   k
+  bf16_t* AsH = Ks + C * QR;                     // [C][SR]   A[t][s] (hi, lo)
   bf16_t* AsL = AsH + C * SR;
   bf16_t* StH = AsL + C * SR;                    // [VT][QR]  the state in front of the chunk, S0[i][j] at [j][i]
   bf16_t* StL = StH + VT * QR;
-  float* pw = reinterpret_cast<float*>(StL + VT * QR);   // [C + 1] powers of the decay
+  bf16_t* last = MODE == 1 ? KtL + DKP * SR : StL + VT * QR;
+  float* pw = reinterpret_cast<float*>(last);    // [C + 1] powers of the decay
 
-  const int seg = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * VT;
+  const int seg = chunks[2 * blockIdx.x], c0 = chunks[2 * blockIdx.x + 1];
+  const int h = blockIdx.y, j0 = blockIdx.z * VT;
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const int li = lane % 16, lc = lane / 16;
-  const int r0 = seg_row0[seg], n = seg_rows[seg];
-  float* S = state + (((size_t)slots[seg] * H + h) * dk) * dv;
+  const int r0 = seg_row0[seg] + c0, nc = min(C, seg_rows[seg] - c0);
+  float* W = ws + (((size_t)blockIdx.x * H + h) * dk) * dv;
   const double lam = (double)decay[h];
 
   {
@@ -73,52 +81,48 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
     for (int i = tid; i < words; i += 256) z[i] = 0u;
   }
   if (tid <= C) pw[tid] = (float)pow(lam, (double)tid);
-
-  floatx4 sreg[IT][4];   // element r: S[i0 + lc * 4 + r][j0 + jt * 16 + li]
-#pragma unroll
-  for (int it = 0; it < IT; ++it)
-#pragma unroll
-    for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = (wave * IT + it) * 16 + lc * 4 + r, j = j0 + jt * 16 + li;
-        sreg[it][jt][r] = (i < dk && j < dv) ? S[(size_t)i * dv + j] : 0.f;
-      }
   __syncthreads();
 
-  for (int c0 = 0; c0 < n; c0 += C) {
-    const int nc = min(C, n - c0);
-    // ---- the state in front of the chunk, as an operand
+  // ---- the chunk's v (both modes), decayed k (1) or q and k (2)
+  for (int idx = tid; idx < C * (VT / 8); idx += 256) {
+    const int s = idx % C, e = (idx / C) * 8;
+    float vv[8];
 #pragma unroll
-    for (int it = 0; it < IT; ++it)
+    for (int x = 0; x < 8; ++x) vv[x] = 0.f;
+    if (s < nc && j0 + e < dv) {
+      unpack8f(load_frag(proj + (size_t)(r0 + s) * ld + v_off + (size_t)h * dv + j0 + e), vv);
+      if (act) {
 #pragma unroll
-      for (int jt = 0; jt < 4; ++jt) {
-        const int at = (jt * 16 + li) * QR + (wave * IT + it) * 16 + lc * 4;
-        store_split4(StH + at, StL + at, sreg[it][jt][0], sreg[it][jt][1], sreg[it][jt][2], sreg[it][jt][3]);
+        for (int x = 0; x < 8; ++x) vv[x] = silu_f(vv[x]);
       }
-    // ---- the chunk's q, k, v
-    for (int idx = tid; idx < C * (DKP / 8); idx += 256) {
-      const int s = idx % C, e = (idx / C) * 8;
-      float qv[8], kv[8];
+    }
 #pragma unroll
-      for (int x = 0; x < 8; ++x) qv[x] = kv[x] = 0.f;
-      if (s < nc && e < dk) {
-        const bf16_t* row = proj + (size_t)(r0 + c0 + s) * ld + (size_t)h * dk + e;
-        unpack8f(load_frag(row + q_off), qv);
-        unpack8f(load_frag(row + k_off), kv);
-        if (act) {
+    for (int x = 0; x < 8; ++x) Vt[(e + x) * SR + s] = float_to_bf16(vv[x]);
+  }
+  for (int idx = tid; idx < C * (DKP / 8); idx += 256) {
+    const int s = idx % C, e = (idx / C) * 8;
+    float qv[8], kv[8];
 #pragma unroll
-          for (int x = 0; x < 8; ++x) { qv[x] = silu_f(qv[x]); kv[x] = silu_f(kv[x]); }
-        }
+    for (int x = 0; x < 8; ++x) qv[x] = kv[x] = 0.f;
+    if (s < nc && e < dk) {
+      const bf16_t* row = proj + (size_t)(r0 + s) * ld + (size_t)h * dk + e;
+      if (MODE == 2) unpack8f(load_frag(row + q_off), qv);
+      unpack8f(load_frag(row + k_off), kv);
+      if (act) {
+#pragma unroll
+        for (int x = 0; x < 8; ++x) { qv[x] = silu_f(qv[x]); kv[x] = silu_f(kv[x]); }
       }
-      Frag fq, fk;
+    }
+    Frag fq, fk;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        fq.w[w] = pack_bf16x2(qv[2 * w], qv[2 * w + 1]);
-        fk.w[w] = pack_bf16x2(kv[2 * w], kv[2 * w + 1]);
-      }
+    for (int w = 0; w < 4; ++w) {
+      fq.w[w] = pack_bf16x2(qv[2 * w], qv[2 * w + 1]);
+      fk.w[w] = pack_bf16x2(kv[2 * w], kv[2 * w + 1]);
+    }
+    if (MODE == 2) {
       *reinterpret_cast<Frag*>(Qs + s * QR + e) = fq;
       *reinterpret_cast<Frag*>(Ks + s * QR + e) = fk;
+    } else {
       const float d = s < nc ? pw[nc - 1 - s] : 0.f;
       float kr[8];
       unpack8f(fk, kr);                       // the rounded keys, as the scores see them
@@ -130,21 +134,51 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
         KtL[(e + x) * SR + s] = float_to_bf16(kd - bf16_to_float(hi));
       }
     }
-    for (int idx = tid; idx < C * (VT / 8); idx += 256) {
-      const int s = idx % C, e = (idx / C) * 8;
-      float vv[8];
+  }
+
+  if constexpr (MODE == 1) {
+    __syncthreads();
+    // ---- tile rows key elements i (the wave's own), columns j
 #pragma unroll
-      for (int x = 0; x < 8; ++x) vv[x] = 0.f;
-      if (s < nc && j0 + e < dv) {
-        unpack8f(load_frag(proj + (size_t)(r0 + c0 + s) * ld + v_off + (size_t)h * dv + j0 + e), vv);
-        if (act) {
+    for (int it = 0; it < IT; ++it) {
+      const int i = (wave * IT + it) * 16 + li;
+      Frag kh[2], kl[2];
 #pragma unroll
-          for (int x = 0; x < 8; ++x) vv[x] = silu_f(vv[x]);
-        }
+      for (int kk = 0; kk < 2; ++kk) {
+        kh[kk] = *reinterpret_cast<const Frag*>(KtH + i * SR + kk * 32 + lc * 8);
+        kl[kk] = *reinterpret_cast<const Frag*>(KtL + i * SR + kk * 32 + lc * 8);
       }
 #pragma unroll
-      for (int x = 0; x < 8; ++x) Vt[(e + x) * SR + s] = float_to_bf16(vv[x]);
+      for (int jt = 0; jt < 4; ++jt) {
+        floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          const Frag vf = *reinterpret_cast<const Frag*>(Vt + (jt * 16 + li) * SR + kk * 32 + lc * 8);
+          acc = mfma16(kh[kk], vf, acc);
+          acc = mfma16(kl[kk], vf, acc);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {      // element r: [i0 + lc * 4 + r][j0 + jt * 16 + li]
+          const int ii = (wave * IT + it) * 16 + lc * 4 + r, j = j0 + jt * 16 + li;
+          if (ii < dk && j < dv) W[(size_t)ii * dv + j] = acc[r];
+        }
+      }
     }
+  } else {
+    // ---- the state in front of the chunk, as an operand (S0[i][j] at [j][i], hi and lo)
+#pragma unroll
+    for (int it = 0; it < IT; ++it)
+#pragma unroll
+      for (int jt = 0; jt < 4; ++jt) {
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = (wave * IT + it) * 16 + lc * 4 + r, j = j0 + jt * 16 + li;
+          v[r] = (i < dk && j < dv) ? W[(size_t)i * dv + j] : 0.f;
+        }
+        const int at = (jt * 16 + li) * QR + (wave * IT + it) * 16 + lc * 4;
+        store_split4(StH + at, StL + at, v[0], v[1], v[2], v[3]);
+      }
     __syncthreads();
 
     // ---- scores of the wave's 16 rows t with all 64 rows s, transposed: tile rows s, columns t
@@ -163,8 +197,8 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int s = st * 16 + lc * 4 + r;
-          acc[r] = s <= t ? acc[r] * pw[t - s] : 0.f;
+          const int s_ = st * 16 + lc * 4 + r;
+          acc[r] = s_ <= t ? acc[r] * pw[t - s_] : 0.f;
         }
       }
       const int at = t * SR + st * 16 + lc * 4;
@@ -173,7 +207,7 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
     wave_lds_order();
 
     // ---- outputs of the wave's rows, transposed: tile rows value columns j, columns t
-    const float from_state = pw[min(t, C - 1) + 1];
+    const float from_state = pw[t + 1];
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt) {
       floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -195,50 +229,43 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
       }
       const int j = j0 + jt * 16 + lc * 4;
       if (t < nc && j < dv)
-        *reinterpret_cast<float4*>(out + (size_t)(r0 + c0 + t) * ldo + (size_t)h * dv + j) =
+        *reinterpret_cast<float4*>(out + (size_t)(r0 + t) * ldo + (size_t)h * dv + j) =
             float4{acc[0], acc[1], acc[2], acc[3]};
     }
-
-    // ---- the state behind the chunk: tile rows key elements i (the wave's own), columns j
-    const float keep = pw[nc];
-#pragma unroll
-    for (int it = 0; it < IT; ++it) {
-      const int i = (wave * IT + it) * 16 + li;
-      Frag kh[2], kl[2];
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        kh[kk] = *reinterpret_cast<const Frag*>(KtH + i * SR + kk * 32 + lc * 8);
-        kl[kk] = *reinterpret_cast<const Frag*>(KtL + i * SR + kk * 32 + lc * 8);
-      }
-#pragma unroll
-      for (int jt = 0; jt < 4; ++jt) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) sreg[it][jt][r] *= keep;
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-          const Frag vf = *reinterpret_cast<const Frag*>(Vt + (jt * 16 + li) * SR + kk * 32 + lc * 8);
-          sreg[it][jt] = mfma16(kh[kk], vf, sreg[it][jt]);
-          sreg[it][jt] = mfma16(kl[kk], vf, sreg[it][jt]);
-        }
-      }
-    }
-    __syncthreads();     // every wave has read this chunk's operands before the next chunk's are written
   }
-
-#pragma unroll
-  for (int it = 0; it < IT; ++it)
-#pragma unroll
-    for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = (wave * IT + it) * 16 + lc * 4 + r, j = j0 + jt * 16 + li;
-        if (i < dk && j < dv) S[(size_t)i * dv + j] = sreg[it][jt][r];
-      }
 }
 
-template <int DKP>
+// Between the two: every element of a request's state walks its segment's chunks in order.  `ws` holds a chunk's
+// contribution U_c on the way in and the state in front of the chunk on the way out: S <- lam^(rows of c) S + U_c.
+// seg_chunks [segments][2]: a segment's first chunk and its chunks.
+__global__ __launch_bounds__(256) void linear_attention_scan_kernel(float* __restrict__ ws, float* __restrict__ state,
+                                                                    const float* __restrict__ decay,
+                                                                    const int* __restrict__ seg_chunks,
+                                                                    const int* __restrict__ seg_rows,
+                                                                    const int* __restrict__ slots, int H, int dk,
+                                                                    int dv) {
+  const int seg = blockIdx.y, per_head = dk * dv;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= H * per_head) return;
+  const int h = idx / per_head;
+  const int first = seg_chunks[2 * seg], n = seg_chunks[2 * seg + 1], rows = seg_rows[seg];
+  const double lam = (double)decay[h];
+  const float whole = (float)pow(lam, (double)C), rest = (float)pow(lam, (double)(rows - (n - 1) * C));
+  float* S = state + (size_t)slots[seg] * H * per_head + idx;
+  float s = *S;
+  for (int c = 0; c < n; ++c) {
+    float* w = ws + (size_t)(first + c) * H * per_head + idx;
+    const float u = *w;
+    *w = s;
+    s = fmaf(c + 1 < n ? whole : rest, s, u);
+  }
+  *S = s;
+}
+
+template <int DKP, int MODE>
 constexpr size_t lds_bytes() {
-  return (size_t)(2 * C * (DKP + PAD) + VT * SR + 2 * DKP * SR + 2 * C * SR + 2 * VT * (DKP + PAD)) * 2 + (C + 1) * 4;
+  return (MODE == 1 ? (size_t)(VT * SR + 2 * DKP * SR) : (size_t)(VT * SR + 2 * C * (DKP + PAD) + 2 * C * SR + 2 * VT * (DKP + PAD))) * 2 +
+         (C + 1) * 4;
 }
 
 }  // namespace
@@ -249,32 +276,42 @@ APC_EXPORT int apc_linear_attention_bf16_takes(int ld, int q_off, int k_off, int
   return 1;
 }
 
+// chunks: int32 [n_chunks][2] (segment, first row of the chunk in it), all segments' chunks in order; seg_chunks: int32
+// [n_segs][2] (a segment's first chunk, its chunks); ws: float32 [n_chunks][H][dk][dv].
 APC_EXPORT int apc_linear_attention_bf16(const void* proj, int ld, int q_off, int k_off, int v_off, int H, int dk,
                                          int dv, int act, const float* decay, float* state, int n_segs,
-                                         const int* seg_row0, const int* seg_rows, const int* slots, float* out,
-                                         int ldo, hipStream_t stream) {
-  if (n_segs <= 0) return 0;
+                                         const int* seg_row0, const int* seg_rows, const int* slots, int n_chunks,
+                                         const int* chunks, const int* seg_chunks, float* ws, float* out, int ldo,
+                                         hipStream_t stream) {
+  if (n_segs <= 0 || n_chunks <= 0) return 0;
   if (!apc_linear_attention_bf16_takes(ld, q_off, k_off, v_off, H, dk, dv)) return APC_ERR_UNSUPPORTED;
-  if (!decay || !state || !slots || ldo < H * dv || ldo % 4 || ((uintptr_t)proj & 15u) || ((uintptr_t)out & 15u))
+  if (!decay || !state || !slots || !chunks || !seg_chunks || !ws || ldo < H * dv || ldo % 4 ||
+      ((uintptr_t)proj & 15u) || ((uintptr_t)out & 15u))
     return APC_ERR_BAD_ARG;
-  dim3 grid(n_segs, H, ceil_div(dv, VT));
-  if (H > 65535 || grid.z > 65535) return APC_ERR_UNSUPPORTED;
-#define LAC_LAUNCH(DKP_)                                                                                            \
+  dim3 grid(n_chunks, H, ceil_div(dv, VT));
+  if (H > 65535 || grid.z > 65535 || n_segs > 65535) return APC_ERR_UNSUPPORTED;
+#define LAC_LAUNCH(DKP_, MODE_)                                                                                     \
   do {                                                                                                              \
-    static bool set_##DKP_ = false;                                                                                 \
-    if (!set_##DKP_) {                                                                                              \
-      hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_attention_chunk_kernel<DKP_>),      \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes<DKP_>());      \
+    static bool set_ = false;                                                                                       \
+    if (!set_) {                                                                                                    \
+      hipError_t e_ = hipFuncSetAttribute(                                                                          \
+          reinterpret_cast<const void*>(&linear_attention_chunk_kernel<DKP_, MODE_>),                               \
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes<DKP_, MODE_>());                               \
       if (e_ != hipSuccess) return (int)e_;                                                                         \
-      set_##DKP_ = true;                                                                                            \
+      set_ = true;                                                                                                  \
     }                                                                                                               \
-    hipLaunchKernelGGL(linear_attention_chunk_kernel<DKP_>, grid, dim3(256), lds_bytes<DKP_>(), stream,             \
-                       (const bf16_t*)proj, ld, q_off, k_off, v_off, H, dk, dv, act, decay, state, seg_row0,        \
-                       seg_rows, slots, out, ldo);                                                                  \
+    hipLaunchKernelGGL((linear_attention_chunk_kernel<DKP_, MODE_>), grid, dim3(256), (lds_bytes<DKP_, MODE_>()),   \
+                       stream, (const bf16_t*)proj, ld, q_off, k_off, v_off, H, dk, dv, act, decay, chunks, ws,     \
+                       seg_row0, seg_rows, out, ldo);                                                               \
+    APC_LAUNCH_CHECK();                                                                                             \
   } while (0)
-  if (dk <= 64) LAC_LAUNCH(64);
-  else LAC_LAUNCH(128);
-#undef LAC_LAUNCH
+  if (dk <= 64) LAC_LAUNCH(64, 1);
+  else LAC_LAUNCH(128, 1);
+  hipLaunchKernelGGL(linear_attention_scan_kernel, dim3(ceil_div(H * dk * dv, 256), n_segs), dim3(256), 0, stream, ws,
+                     state, decay, seg_chunks, seg_rows, slots, H, dk, dv);
   APC_LAUNCH_CHECK();
+  if (dk <= 64) LAC_LAUNCH(64, 2);
+  else LAC_LAUNCH(128, 2);
+#undef LAC_LAUNCH
   return 0;
 }

@@ -80,7 +80,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_routed_max_tiles": [I, I, I],
         "apc_routed_experts_bf16": [P, I, P, P, I, I, I, P, P, I, I, I, P, P, P, P, P, I, P],
         "apc_linear_attention_bf16_takes": [I, I, I, I, I, I, I],
-        "apc_linear_attention_bf16": [P, I, I, I, I, I, I, I, I, P, P, I, P, P, P, P, I, P],
+        "apc_linear_attention_bf16": [P, I, I, I, I, I, I, I, I, P, P, I, P, P, P, I, P, P, P, P, I, P],
         "apc_attention_masked_takes": [I, I, I, I, I, I],
         "apc_attention_masked_prefill_bf16": [P, I, P, I, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, F, I, I, P],
         "apc_attention_masked_decode_bf16": [P, I, P, I, I, I, I, I, I, P, I, P, I, P, P, P, I, I, I, F, I, P, I, I, P],

@@ -518,11 +518,35 @@ def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, sta
             or not L.apc_linear_attention_bf16_takes(ld, q_off, k_off, v_off, H, dk, dv)):
         return False
     S = step.n_segs
+    n_chunks, chunks, seg_chunks = _row_chunks(step, proj.device)
+    ws = torch.empty((n_chunks, H, dk, dv), dtype=torch.float32, device=proj.device)
     _lib.check(L.apc_linear_attention_bf16(
         proj.data_ptr(), ld, q_off, k_off, v_off, H, dk, dv, 1 if silu else 0, _ops._f32(decay, H, "decay"),
         state.data_ptr(), S, _ops._i32(step.seg_row0, S, "seg_row0"), _ops._i32(step.seg_rows, S, "seg_rows"),
-        _ops._i32(slots, S, "slots"), out.data_ptr(), ldo, _ops._stream()), "linear_attention_bf16")
+        _ops._i32(slots, S, "slots"), n_chunks, chunks.data_ptr(), seg_chunks.data_ptr(), ws.data_ptr(),
+        out.data_ptr(), ldo, _ops._stream()), "linear_attention_bf16")
     return True
+
+
+LINEAR_CHUNK_ROWS = 64
+
+
+def _row_chunks(step, device):
+    """(chunks in all, int32 [chunks][2] (segment, first row in it), int32 [segments][2] (a segment's first chunk, its
+    chunks)) of a step's segments cut into chunks of 64 rows: made on the host from the step's own lists, once a step
+    (every layer of the step asks for the same)."""
+    made = getattr(step, "_row_chunks", None)
+    if made is None:
+        import numpy as np
+        chunks, per_seg = [], []
+        for s, n in enumerate(step.host_rows):
+            per_seg.append((len(chunks), -(-n // LINEAR_CHUNK_ROWS)))
+            chunks += [(s, c0) for c0 in range(0, n, LINEAR_CHUNK_ROWS)]
+        flat = np.asarray(chunks + per_seg, dtype=np.int32).reshape(-1)
+        dev = torch.from_numpy(flat).to(device)
+        made = (len(chunks), dev[:2 * len(chunks)], dev[2 * len(chunks):])
+        step._row_chunks = made
+    return made
 
 
 class PackedExperts:
