@@ -48,7 +48,7 @@ __device__ __forceinline__ void store_split4(bf16_t* ph, bf16_t* pl, float a, fl
 template <int DKP, int MODE>  // key size rounded up to a multiple of 64
 __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
     const bf16_t* __restrict__ proj, int ld, int q_off, int k_off, int v_off, int H, int dk, int dv, int act,
-    const float* __restrict__ decay, const int* __restrict__ chunks, float* __restrict__ ws,
+    const float* __restrict__ powers, const int* __restrict__ chunks, float* __restrict__ ws,
     const int* __restrict__ seg_row0, const int* __restrict__ seg_rows, float* __restrict__ out, int ldo) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   constexpr int QR = DKP + PAD;
@@ -58,8 +58,7 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
   bf16_t* KtH = Vt + VT * SR;                    // [DKP][SR] decayed k, a key element's rows side by side (hi, lo)
   bf16_t* KtL = KtH + DKP * SR;
   // MODE 2
-  bf16_t* Qs = Vt + VT * SR;                     // [C][QR]   q of the chunk's rows
-  bf16_t* Ks = Qs + C * QR;                      // [C][QR]   k
+  bf16_t* Ks = Vt + VT * SR;                     // [C][QR]   k of the chunk's rows
   bf16_t* AsH = Ks + C * QR;                     // [C][SR]   A[t][s] (hi, lo)
   bf16_t* AsL = AsH + C * SR;
   bf16_t* StH = AsL + C * SR;                    // [VT][QR]  the state in front of the chunk, S0[i][j] at [j][i]
@@ -73,17 +72,12 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
   const int li = lane % 16, lc = lane / 16;
   const int r0 = seg_row0[seg] + c0, nc = min(C, seg_rows[seg] - c0);
   float* W = ws + (((size_t)blockIdx.x * H + h) * dk) * dv;
-  const double lam = (double)decay[h];
-
-  {
-    uint32_t* z = reinterpret_cast<uint32_t*>(lds);
-    const int words = (int)((reinterpret_cast<unsigned char*>(pw) - lds) / 4);
-    for (int i = tid; i < words; i += 256) z[i] = 0u;
-  }
-  if (tid <= C) pw[tid] = (float)pow(lam, (double)tid);
+  // (every element of LDS that is read below is written below: rows beyond the chunk's and columns beyond the sizes
+  // as zeros)
+  if (tid <= C) pw[tid] = powers[(size_t)h * (C + 1) + tid];
   __syncthreads();
 
-  // ---- the chunk's v (both modes), decayed k (1) or q and k (2)
+  // ---- the chunk's v (both modes), decayed k (1) or k (2)
   for (int idx = tid; idx < C * (VT / 8); idx += 256) {
     const int s = idx % C, e = (idx / C) * 8;
     float vv[8];
@@ -101,26 +95,20 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
   }
   for (int idx = tid; idx < C * (DKP / 8); idx += 256) {
     const int s = idx % C, e = (idx / C) * 8;
-    float qv[8], kv[8];
+    float kv[8];
 #pragma unroll
-    for (int x = 0; x < 8; ++x) qv[x] = kv[x] = 0.f;
+    for (int x = 0; x < 8; ++x) kv[x] = 0.f;
     if (s < nc && e < dk) {
-      const bf16_t* row = proj + (size_t)(r0 + s) * ld + (size_t)h * dk + e;
-      if (MODE == 2) unpack8f(load_frag(row + q_off), qv);
-      unpack8f(load_frag(row + k_off), kv);
+      unpack8f(load_frag(proj + (size_t)(r0 + s) * ld + (size_t)h * dk + e + k_off), kv);
       if (act) {
 #pragma unroll
-        for (int x = 0; x < 8; ++x) { qv[x] = silu_f(qv[x]); kv[x] = silu_f(kv[x]); }
+        for (int x = 0; x < 8; ++x) kv[x] = silu_f(kv[x]);
       }
     }
-    Frag fq, fk;
+    Frag fk;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      fq.w[w] = pack_bf16x2(qv[2 * w], qv[2 * w + 1]);
-      fk.w[w] = pack_bf16x2(kv[2 * w], kv[2 * w + 1]);
-    }
+    for (int w = 0; w < 4; ++w) fk.w[w] = pack_bf16x2(kv[2 * w], kv[2 * w + 1]);
     if (MODE == 2) {
-      *reinterpret_cast<Frag*>(Qs + s * QR + e) = fq;
       *reinterpret_cast<Frag*>(Ks + s * QR + e) = fk;
     } else {
       const float d = s < nc ? pw[nc - 1 - s] : 0.f;
@@ -183,9 +171,24 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
 
     // ---- scores of the wave's 16 rows t with all 64 rows s, transposed: tile rows s, columns t
     const int t = wave * 16 + li;              // the lane's row of the chunk as a column of the tiles
+    // (its q as the second operand of every product comes straight from memory: no other wave needs it)
     Frag qf[DKP / 32];
 #pragma unroll
-    for (int ks = 0; ks < DKP / 32; ++ks) qf[ks] = *reinterpret_cast<const Frag*>(Qs + t * QR + ks * 32 + lc * 8);
+    for (int ks = 0; ks < DKP / 32; ++ks) {
+      const int e = ks * 32 + lc * 8;
+      float qv[8];
+#pragma unroll
+      for (int x = 0; x < 8; ++x) qv[x] = 0.f;
+      if (t < nc && e < dk) {
+        unpack8f(load_frag(proj + (size_t)(r0 + t) * ld + (size_t)h * dk + e + q_off), qv);
+        if (act) {
+#pragma unroll
+          for (int x = 0; x < 8; ++x) qv[x] = silu_f(qv[x]);
+        }
+      }
+#pragma unroll
+      for (int w = 0; w < 4; ++w) qf[ks].w[w] = pack_bf16x2(qv[2 * w], qv[2 * w + 1]);
+    }
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
       floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -239,7 +242,7 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
 // contribution U_c on the way in and the state in front of the chunk on the way out: S <- lam^(rows of c) S + U_c.
 // seg_chunks [segments][2]: a segment's first chunk and its chunks.
 __global__ __launch_bounds__(256) void linear_attention_scan_kernel(float* __restrict__ ws, float* __restrict__ state,
-                                                                    const float* __restrict__ decay,
+                                                                    const float* __restrict__ powers,
                                                                     const int* __restrict__ seg_chunks,
                                                                     const int* __restrict__ seg_rows,
                                                                     const int* __restrict__ slots, int H, int dk,
@@ -249,8 +252,7 @@ __global__ __launch_bounds__(256) void linear_attention_scan_kernel(float* __res
   if (idx >= H * per_head) return;
   const int h = idx / per_head;
   const int first = seg_chunks[2 * seg], n = seg_chunks[2 * seg + 1], rows = seg_rows[seg];
-  const double lam = (double)decay[h];
-  const float whole = (float)pow(lam, (double)C), rest = (float)pow(lam, (double)(rows - (n - 1) * C));
+  const float whole = powers[(size_t)h * (C + 1) + C], rest = powers[(size_t)h * (C + 1) + rows - (n - 1) * C];
   float* S = state + (size_t)slots[seg] * H * per_head + idx;
   float s = *S;
   for (int c = 0; c < n; ++c) {
@@ -264,7 +266,7 @@ __global__ __launch_bounds__(256) void linear_attention_scan_kernel(float* __res
 
 template <int DKP, int MODE>
 constexpr size_t lds_bytes() {
-  return (MODE == 1 ? (size_t)(VT * SR + 2 * DKP * SR) : (size_t)(VT * SR + 2 * C * (DKP + PAD) + 2 * C * SR + 2 * VT * (DKP + PAD))) * 2 +
+  return (MODE == 1 ? (size_t)(VT * SR + 2 * DKP * SR) : (size_t)(VT * SR + C * (DKP + PAD) + 2 * C * SR + 2 * VT * (DKP + PAD))) * 2 +
          (C + 1) * 4;
 }
 
@@ -276,16 +278,17 @@ APC_EXPORT int apc_linear_attention_bf16_takes(int ld, int q_off, int k_off, int
   return 1;
 }
 
+// powers: float32 [H][65], decay[h]^0 .. decay[h]^64 (rounded from double precision once, by the caller).
 // chunks: int32 [n_chunks][2] (segment, first row of the chunk in it), all segments' chunks in order; seg_chunks: int32
 // [n_segs][2] (a segment's first chunk, its chunks); ws: float32 [n_chunks][H][dk][dv].
 APC_EXPORT int apc_linear_attention_bf16(const void* proj, int ld, int q_off, int k_off, int v_off, int H, int dk,
-                                         int dv, int act, const float* decay, float* state, int n_segs,
+                                         int dv, int act, const float* powers, float* state, int n_segs,
                                          const int* seg_row0, const int* seg_rows, const int* slots, int n_chunks,
                                          const int* chunks, const int* seg_chunks, float* ws, float* out, int ldo,
                                          hipStream_t stream) {
   if (n_segs <= 0 || n_chunks <= 0) return 0;
   if (!apc_linear_attention_bf16_takes(ld, q_off, k_off, v_off, H, dk, dv)) return APC_ERR_UNSUPPORTED;
-  if (!decay || !state || !slots || !chunks || !seg_chunks || !ws || ldo < H * dv || ldo % 4 ||
+  if (!powers || !state || !slots || !chunks || !seg_chunks || !ws || ldo < H * dv || ldo % 4 ||
       ((uintptr_t)proj & 15u) || ((uintptr_t)out & 15u))
     return APC_ERR_BAD_ARG;
   dim3 grid(n_chunks, H, ceil_div(dv, VT));
@@ -301,14 +304,14 @@ APC_EXPORT int apc_linear_attention_bf16(const void* proj, int ld, int q_off, in
       set_ = true;                                                                                                  \
     }                                                                                                               \
     hipLaunchKernelGGL((linear_attention_chunk_kernel<DKP_, MODE_>), grid, dim3(256), (lds_bytes<DKP_, MODE_>()),   \
-                       stream, (const bf16_t*)proj, ld, q_off, k_off, v_off, H, dk, dv, act, decay, chunks, ws,     \
+                       stream, (const bf16_t*)proj, ld, q_off, k_off, v_off, H, dk, dv, act, powers, chunks, ws,    \
                        seg_row0, seg_rows, out, ldo);                                                               \
     APC_LAUNCH_CHECK();                                                                                             \
   } while (0)
   if (dk <= 64) LAC_LAUNCH(64, 1);
   else LAC_LAUNCH(128, 1);
   hipLaunchKernelGGL(linear_attention_scan_kernel, dim3(ceil_div(H * dk * dv, 256), n_segs), dim3(256), 0, stream, ws,
-                     state, decay, seg_chunks, seg_rows, slots, H, dk, dv);
+                     state, powers, seg_chunks, seg_rows, slots, H, dk, dv);
   APC_LAUNCH_CHECK();
   if (dk <= 64) LAC_LAUNCH(64, 2);
   else LAC_LAUNCH(128, 2);

@@ -24,6 +24,7 @@ namespace {
 
 constexpr int TILE_ELEMS = 512;
 constexpr int MAX_EXPERTS = 1024;
+constexpr int STREAM_U = 4;       // chunks of 32 columns a wave asks for together
 
 __global__ __launch_bounds__(1024) void routed_sort_kernel(const int* __restrict__ ids, int n_pairs, int E,
                                                            int tile_rows, int* __restrict__ order,
@@ -72,7 +73,8 @@ __global__ __launch_bounds__(1024) void routed_sort_kernel(const int* __restrict
   }
 }
 
-// RT tiles of 16 rows a wave: a weight tile read from memory feeds RT MFMAs
+// RT tiles of 16 rows a wave: a weight tile read from memory feeds RT MFMAs (the launches use 1: more rows an expert
+// go to the tiled kernel)
 template <int RT>
 __global__ __launch_bounds__(256) void routed_glu_bf16_kernel(const bf16_t* __restrict__ h, int ldh,
                                                               const bf16_t* __restrict__ w_gate_up, int F, int D,
@@ -100,11 +102,33 @@ __global__ __launch_bounds__(256) void routed_glu_bf16_kernel(const bf16_t* __re
   floatx4 g[RT], u[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) g[rt] = u[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  for (int c = 0; c < chunks; ++c) {
-    const Frag fg = load_frag(wg + (size_t)c * TILE_ELEMS), fu = load_frag(wu + (size_t)c * TILE_ELEMS);
+  // The weights are read once a tile: loads that the caches do not keep, STREAM_U chunks asked for together so that a
+  // wave has 8 KiB of them in flight (one chunk at a time a wave waited a trip to memory for every 2 KiB).
+  int c = 0;
+  for (; c + STREAM_U <= chunks; c += STREAM_U) {
+    Frag fg[STREAM_U], fu[STREAM_U], a[STREAM_U][RT];
+#pragma unroll
+    for (int x = 0; x < STREAM_U; ++x) {
+      fg[x] = load_frag_once(wg + (size_t)(c + x) * TILE_ELEMS);
+      fu[x] = load_frag_once(wu + (size_t)(c + x) * TILE_ELEMS);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+        // (a last chunk that reaches beyond D: the weights' tile is zero there, the row's elements must not be read)
+        a[x][rt] = (on[rt] && (c + x < full || (c + x) * 32 + lc * 8 < D)) ? load_frag(arow[rt] + (c + x) * 32)
+                                                                          : zero_frag();
+    }
+#pragma unroll
+    for (int x = 0; x < STREAM_U; ++x)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        g[rt] = mfma16(fg[x], a[x][rt], g[rt]);
+        u[rt] = mfma16(fu[x], a[x][rt], u[rt]);
+      }
+  }
+  for (; c < chunks; ++c) {
+    const Frag fg = load_frag_once(wg + (size_t)c * TILE_ELEMS), fu = load_frag_once(wu + (size_t)c * TILE_ELEMS);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      // (a last chunk that reaches beyond D: the weights' tile is zero there, the row's elements must not be read)
       const Frag a = (on[rt] && (c < full || c * 32 + lc * 8 < D)) ? load_frag(arow[rt] + c * 32) : zero_frag();
       g[rt] = mfma16(fg, a, g[rt]);
       u[rt] = mfma16(fu, a, u[rt]);
@@ -155,8 +179,24 @@ __global__ __launch_bounds__(256) void routed_down_bf16_kernel(const bf16_t* __r
   floatx4 acc[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) acc[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  for (int c = 0; c < chunks; ++c) {
-    const Frag fw = load_frag(wd + (size_t)c * TILE_ELEMS);
+  int c = 0;
+  for (; c + 2 * STREAM_U <= chunks; c += 2 * STREAM_U) {
+    Frag fw[2 * STREAM_U], a[2 * STREAM_U][RT];
+#pragma unroll
+    for (int x = 0; x < 2 * STREAM_U; ++x) {
+      fw[x] = load_frag_once(wd + (size_t)(c + x) * TILE_ELEMS);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+        a[x][rt] = (on[rt] && (c + x < full || (c + x) * 32 + lc * 8 < F)) ? load_frag(arow[rt] + (c + x) * 32)
+                                                                          : zero_frag();
+    }
+#pragma unroll
+    for (int x = 0; x < 2 * STREAM_U; ++x)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) acc[rt] = mfma16(fw[x], a[x][rt], acc[rt]);
+  }
+  for (; c < chunks; ++c) {
+    const Frag fw = load_frag_once(wd + (size_t)c * TILE_ELEMS);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       const Frag a = (on[rt] && (c < full || c * 32 + lc * 8 < F)) ? load_frag(arow[rt] + c * 32) : zero_frag();
@@ -183,7 +223,7 @@ __global__ __launch_bounds__(256) void routed_gather_kernel(const bf16_t* __rest
   if (ti >= *n_tiles) return;
   const int p0 = tiles[3 * ti + 1], rows = tiles[3 * ti + 2];
   const int pieces = D / 8;
-  for (int idx = threadIdx.x; idx < rows * pieces; idx += 256) {
+  for (int idx = blockIdx.y * 256 + threadIdx.x; idx < rows * pieces; idx += gridDim.y * 256) {
     const int r = idx / pieces, c = (idx % pieces) * 8;
     *reinterpret_cast<Frag*>(hs + (size_t)(p0 + r) * D + c) = load_frag(h + (size_t)(order[p0 + r] / K) * ldh + c);
   }
@@ -254,7 +294,7 @@ APC_EXPORT int apc_routed_experts_bf16(const void* h, int ldh, const void* w_gat
     APC_LAUNCH_CHECK();
   } else {
     if (max_tiles > 65535) return APC_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(routed_gather_kernel, dim3(max_tiles), dim3(256), 0, stream, (const bf16_t*)h, ldh, D, order, K,
+    hipLaunchKernelGGL(routed_gather_kernel, dim3(max_tiles, 16), dim3(256), 0, stream, (const bf16_t*)h, ldh, D, order, K,
                        tiles, n_tiles, tile_rows, (bf16_t*)hs);
     APC_LAUNCH_CHECK();
     const size_t gate_elems = (size_t)ceil_div(F, 16) * ceil_div(D, 32) * TILE_ELEMS;

@@ -521,7 +521,8 @@ def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, sta
     n_chunks, chunks, seg_chunks = _row_chunks(step, proj.device)
     ws = torch.empty((n_chunks, H, dk, dv), dtype=torch.float32, device=proj.device)
     _lib.check(L.apc_linear_attention_bf16(
-        proj.data_ptr(), ld, q_off, k_off, v_off, H, dk, dv, 1 if silu else 0, _ops._f32(decay, H, "decay"),
+        proj.data_ptr(), ld, q_off, k_off, v_off, H, dk, dv, 1 if silu else 0,
+        _ops._f32(_decay_powers(decay), H * (LINEAR_CHUNK_ROWS + 1), "powers of the decay"),
         state.data_ptr(), S, _ops._i32(step.seg_row0, S, "seg_row0"), _ops._i32(step.seg_rows, S, "seg_rows"),
         _ops._i32(slots, S, "slots"), n_chunks, chunks.data_ptr(), seg_chunks.data_ptr(), ws.data_ptr(),
         out.data_ptr(), ldo, _ops._stream()), "linear_attention_bf16")
@@ -529,6 +530,18 @@ def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, sta
 
 
 LINEAR_CHUNK_ROWS = 64
+_POWERS: dict = {}
+
+
+def _decay_powers(decay: torch.Tensor) -> torch.Tensor:
+    """float32 [heads, 65]: decay^0 .. decay^64 of every head, formed in double precision, once for a decay tensor."""
+    key = (decay.data_ptr(), decay.numel(), decay.device)
+    made = _POWERS.get(key)
+    if made is None or made[0] is not decay:
+        n = torch.arange(LINEAR_CHUNK_ROWS + 1, dtype=torch.float64, device=decay.device)
+        made = (decay, torch.pow(decay.double()[:, None], n[None, :]).float().contiguous())
+        _POWERS[key] = made
+    return made[1]
 
 
 def _row_chunks(step, device):

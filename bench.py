@@ -73,6 +73,8 @@ def weight_bytes(eng):
         nonlocal total
         if isinstance(v, PackedWeight):
             v = v.data
+        elif not isinstance(v, torch.Tensor) and isinstance(getattr(v, "data", None), torch.Tensor):
+            v = v.data          # (the tiled matrices of a layer's experts)
         if isinstance(v, (tuple, list)):
             for x in v:
                 add(x)
@@ -510,12 +512,14 @@ def gulidra_rooflines(size, batch, context, T, points):
             return rows * (att_own * (own + q + 2 * G * d) + (att_all - att_own) * 2 * q) * 2, 0
         if name in ("apc_rope_kv_write_bf16", "apc_rope_kv_write"):
             return layers * rows * ((H + 2 * G) * d + H * d + 2 * G * d) * 2, 0
-        if name in ("apc_attention_masked_prefill_bf16", "apc_attention_prefill_bf16"):
+        if name == "apc_attention_masked_prefill_bf16":      # two maps of d / 2 a head, each over values of d
+            return 0, att_all * keys_sum * H * 2 * (2 * (d // 2) + 2 * d)
+        if name == "apc_attention_prefill_bf16":
             return 0, att_all * 4 * keys_sum * H * d
         if name in ("apc_attention_masked_decode_bf16", "apc_attention_decode_bf16"):
             return att_all * keys_sum * G * 2 * d * 2, 0
-        if name == "apc_linear_attention_bf16":      # scores and their use inside chunks of 64, state read and moved on
-            return 0, lin * rows * H * (2 * 64 * d + 2 * 64 * d + 4 * d * d) // 2 * 2
+        if name == "apc_linear_attention_bf16":      # a row: scores with and weights over half a chunk of 64 on
+            return 0, lin * rows * H * 2 * (32 * d + 32 * d + 2 * d * d)      # average, the state read and moved on
         if name == "apc_linear_attention":           # the state of every row read and written
             return lin * rows * H * d * d * 4 * 2, 0
         if name == "apc_routed_experts_bf16":

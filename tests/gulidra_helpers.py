@@ -68,7 +68,23 @@ TINY_GC = dict(
             _layer(_lin(1, 16, 16, (1.0,)), _moe(24, 3, 0, 3)),
             _layer(_att(1, 1, 16, 16, 0.25, 0.0, conv=0, kv_from=0), None)])
 
-CONFIGS = {"GA": (TINY_GA, 21), "GB": (TINY_GB, 22), "GC": (TINY_GC, 23)}
+# D: recurrent layers only (no pages at all), the first one without feed-forward
+TINY_GD = dict(
+    architecture="Gulidra", vocab=70, width=48, max_positions=200, embedding=dict(scale=0.5), residual_mult=1.5,
+    norm=dict(eps=1e-5),
+    layers=[_layer(_lin(3, 16, 24, (0.9, 0.95, 0.99)), None),
+            _layer(_lin(2, 40, 8, (0.6, 0.999)), _moe(40, 2, 3, 2))])
+# E: a borrower behind recurrent layers, two owners, experts without any identity key
+TINY_GE = dict(
+    architecture="Gulidra", vocab=64, width=64, max_positions=200, embedding=dict(scale=4.0), residual_mult=0.25,
+    norm=dict(eps=1e-6),
+    layers=[_layer(_att(4, 1, 16, 32, 0.25, 0.35, conv=5), _dense(96)),
+            _layer(_lin(2, 32, 32, (0.97, 0.9)), dict(kind="moe", expert=dict(ff=48), router=dict(experts=3, top=1))),
+            _layer(_att(2, 2, 24, 16, 0.2, 0.15, conv=3), None),
+            _layer(_att(4, 1, 16, 32, 0.3, 0.3, conv=2, kv_from=0), _dense(80)),
+            _layer(_att(2, 2, 24, 16, 0.2, 0.6, kv_from=2), _moe(64, 2, 1, 3))])
+
+CONFIGS = {"GA": (TINY_GA, 21), "GB": (TINY_GB, 22), "GC": (TINY_GC, 23), "GD": (TINY_GD, 24), "GE": (TINY_GE, 25)}
 
 
 def planted(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:

@@ -331,7 +331,7 @@ def test_layers_one_by_one_in_32_bit():
             close(np.concatenate([got[i], got[n + i]]), want[i], "float32", f"{name} layer {i}")
 
 
-@pytest.mark.parametrize("name", ["GA", "GB", "GC"])
+@pytest.mark.parametrize("name", ["GA", "GB", "GC", "GD", "GE"])
 @pytest.mark.parametrize("dtype, page_tokens", [("float32", 4), ("bfloat16", 4), ("bfloat16", 16)])
 def test_whole_prompts_decoding_and_portions(name, dtype, page_tokens):
     """(Pages of 16 positions: the bfloat16 run's attention on the matrix-core kernels; of 4: on the plain one.)"""
@@ -365,7 +365,7 @@ def test_first_tokens_and_page_sizes(name):
 
 
 @pytest.mark.parametrize("name, dtype, page_tokens", [("GA", "float32", 4), ("GB", "float32", 4), ("GB", "bfloat16", 16),
-                                                     ("GB", "bfloat16", 8), ("GC", "float32", 4)])
+                                                     ("GB", "bfloat16", 8), ("GC", "float32", 4), ("GE", "bfloat16", 16)])
 def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, page_tokens):
     """Five requests of unequal lengths through three slots and a pool that cannot hold them all at once: portions of
     some beside single tokens of others, free pages filled with a huge number.  A slot that comes back carries the
@@ -475,6 +475,14 @@ def test_command_line_and_replay_program(tmp_path):
     assert r.returncode == 0, r.stderr[-2000:]
     outs = [json.loads(ln) for ln in r.stdout.strip().splitlines() if ln.startswith("{")]
     assert [o["token_ids"] for o in outs] == [P.greedy(oracle(folder), p, 6) for p in prompts]
+    # the design's preset with random weights, sampled with temperature, top-k and top-p in bfloat16
+    cmd = [sys.executable, os.path.join(root, "bin", "allpaca-amd"), "generate", "--synthetic", "gulidra-tiny",
+           "--prompt-tokens", "1,2,3;4,5", "--max-tokens", "5", "--temperature", "0.8", "--top-k", "20", "--top-p",
+           "0.9", "--json"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    outs = [json.loads(ln) for ln in r.stdout.strip().splitlines() if ln.startswith("{")]
+    assert len(outs) == 2 and all(len(o["token_ids"]) == 5 for o in outs)
 
     name = "GB"
     folder = model_folder(name)
