@@ -103,14 +103,16 @@ __global__ __launch_bounds__(256) void routed_down_kernel(const void* __restrict
                                                           int D, const int* __restrict__ ids,
                                                           const float* __restrict__ weights, int K,
                                                           const void* __restrict__ h, int h_dtype, int ldh,
-                                                          float* __restrict__ y, int ldy) {
-  extern __shared__ float as[];        // [K][F]
+                                                          float* __restrict__ y, int ldy, int in_lds) {
+  extern __shared__ float as[];        // [K][F], if the row's activations fit (else they are read where they lie)
   const int t = blockIdx.x;
-  for (int i = threadIdx.x; i < K * F; i += 256) {
-    const int k = i / F;
-    as[i] = ids[(size_t)t * K + k] < E ? load_f(act, act_dtype, (size_t)t * K * F + i) : 0.f;
+  if (in_lds) {
+    for (int i = threadIdx.x; i < K * F; i += 256) {
+      const int k = i / F;
+      as[i] = ids[(size_t)t * K + k] < E ? load_f(act, act_dtype, (size_t)t * K * F + i) : 0.f;
+    }
+    __syncthreads();
   }
-  __syncthreads();
   const int d = blockIdx.y * 256 + threadIdx.x;
   if (d >= D) return;
   float total = 0.f;
@@ -120,7 +122,12 @@ __global__ __launch_bounds__(256) void routed_down_kernel(const void* __restrict
     if (e < E) {
       const size_t row = ((size_t)e * D + d) * F;
       v = 0.f;
-      for (int f = 0; f < F; ++f) v = fmaf(as[k * F + f], load_f(w_down, w_dtype, row + f), v);
+      if (in_lds) {
+        for (int f = 0; f < F; ++f) v = fmaf(as[k * F + f], load_f(w_down, w_dtype, row + f), v);
+      } else {
+        const size_t a0 = ((size_t)t * K + k) * F;
+        for (int f = 0; f < F; ++f) v = fmaf(load_f(act, act_dtype, a0 + f), load_f(w_down, w_dtype, row + f), v);
+      }
     } else {
       v = load_f(h, h_dtype, (size_t)t * ldh + d);
     }
@@ -159,9 +166,11 @@ APC_EXPORT int apc_routed_down(const void* act, int act_dtype, const void* w_dow
                                float* y, int ldy, int n_rows, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (E < 0 || F <= 0 || D <= 0 || K <= 0 || ldh < D || ldy < D) return APC_ERR_BAD_ARG;
-  if ((size_t)K * F * sizeof(float) > 64 * 1024 || ceil_div(D, 256) > 65535) return APC_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(routed_down_kernel, dim3(n_rows, ceil_div(D, 256)), dim3(256), (size_t)K * F * sizeof(float),
-                     stream, act, act_dtype, w_down, w_dtype, E, F, D, ids, weights, K, h, h_dtype, ldh, y, ldy);
+  if (ceil_div(D, 256) > 65535) return APC_ERR_UNSUPPORTED;
+  const size_t lds = (size_t)K * F * sizeof(float);
+  const int in_lds = lds <= 48 * 1024 ? 1 : 0;       // (the same sums in the same order either way)
+  hipLaunchKernelGGL(routed_down_kernel, dim3(n_rows, ceil_div(D, 256)), dim3(256), in_lds ? lds : 0, stream, act,
+                     act_dtype, w_down, w_dtype, E, F, D, ids, weights, K, h, h_dtype, ldh, y, ldy, in_lds);
   APC_LAUNCH_CHECK();
   return 0;
 }

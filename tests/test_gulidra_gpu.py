@@ -227,7 +227,8 @@ def test_router_choice_with_correction(N, K):
 
 
 @pytest.mark.parametrize("D, F, E, I, K, T", [(36, 20, 5, 2, 3, 19), (128, 64, 8, 1, 2, 150), (64, 32, 3, 0, 3, 40),
-                                             (32, 16, 1, 1, 2, 7), (256, 96, 4, 3, 2, 700)])
+                                             (32, 16, 1, 1, 2, 7), (256, 96, 4, 3, 2, 700),
+                                             (32, 4096, 4, 0, 4, 5)])      # a row's activations larger than LDS
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_routed_experts_with_identities(D, F, E, I, K, T, dtype):
     """Few rows (tiles of 16 of the matrix-core kernels, most of them nearly empty) and many (tiles of 64), experts that
