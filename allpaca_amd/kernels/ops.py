@@ -605,11 +605,12 @@ def rmsnorm_add(y: torch.Tensor, weight: torch.Tensor, eps: float, mult: float, 
 # --------------------------------------------------------------------------- linear attention with a decay
 def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: int, key_dim: int,
                      value_dim: int, silu: bool, decay: torch.Tensor, state: torch.Tensor, step, slots: torch.Tensor,
-                     out: torch.Tensor) -> None:
+                     out: torch.Tensor, powers: Optional[torch.Tensor] = None) -> None:
     """Per head S <- decay * S + k_t v_t^T, o_t = S^T q_t over the rows of every segment in order, S float32
     [slots + 1, heads, key_dim, value_dim] per request; q, k, v (through silu if asked) from the projected rows;
-    `out` float32 [rows, heads * value_dim]."""
-    _gpu(proj, decay, state, slots, out)
+    `out` float32 [rows, heads * value_dim].  `powers` (optional): `tuned.decay_powers` of the same decay, kept by the
+    caller for the kernel that walks prompt portions in chunks."""
+    _gpu(proj, decay, state, slots, out, powers)
     ld, ldo = _rows(proj, "projected rows"), _rows(out, "linear attention out")
     T, width = proj.shape
     H, dk, dv = int(n_heads), int(key_dim), int(value_dim)
@@ -621,7 +622,8 @@ def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_h
     S = step.n_segs
     if _tuned_ok(proj):
         from . import tuned
-        if tuned.linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, state, step, slots, out):
+        if tuned.linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, state, step, slots, out,
+                                       powers):
             return
     L = _lib.load("plain")
     _lib.check(L.apc_linear_attention(proj.data_ptr(), _code(proj), ld, q_off, k_off, v_off, H, dk, dv,

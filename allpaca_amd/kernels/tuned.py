@@ -508,7 +508,8 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
 LINEAR_CHUNK_MIN_ROWS = 5    # segments of at least this many rows make a step run on the kernel of 64-row chunks
 
 
-def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, state, step, slots, out) -> bool:
+def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, state, step, slots, out,
+                          powers=None) -> bool:
     """Linear attention with a decay on the MFMA kernel that walks a segment in chunks of 64 rows.  False (nothing
     done) for sizes it does not take and for steps whose segments are all short (decoded rows): the caller then runs
     the kernel that walks row by row."""
@@ -518,11 +519,13 @@ def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, sta
             or not L.apc_linear_attention_bf16_takes(ld, q_off, k_off, v_off, H, dk, dv)):
         return False
     S = step.n_segs
+    if powers is None:         # (a caller that keeps the table, as the mixer does, saves this read-back)
+        powers = decay_powers(decay.tolist(), proj.device)
     n_chunks, chunks, seg_chunks = _row_chunks(step, proj.device)
     ws = torch.empty((n_chunks, H, dk, dv), dtype=torch.float32, device=proj.device)
     _lib.check(L.apc_linear_attention_bf16(
         proj.data_ptr(), ld, q_off, k_off, v_off, H, dk, dv, 1 if silu else 0,
-        _ops._f32(_decay_powers(decay), H * (LINEAR_CHUNK_ROWS + 1), "powers of the decay"),
+        _ops._f32(powers, H * (LINEAR_CHUNK_ROWS + 1), "powers of the decay"),
         state.data_ptr(), S, _ops._i32(step.seg_row0, S, "seg_row0"), _ops._i32(step.seg_rows, S, "seg_rows"),
         _ops._i32(slots, S, "slots"), n_chunks, chunks.data_ptr(), seg_chunks.data_ptr(), ws.data_ptr(),
         out.data_ptr(), ldo, _ops._stream()), "linear_attention_bf16")
@@ -530,18 +533,13 @@ def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, sta
 
 
 LINEAR_CHUNK_ROWS = 64
-_POWERS: dict = {}
 
 
-def _decay_powers(decay: torch.Tensor) -> torch.Tensor:
-    """float32 [heads, 65]: decay^0 .. decay^64 of every head, formed in double precision, once for a decay tensor."""
-    key = (decay.data_ptr(), decay.numel(), decay.device)
-    made = _POWERS.get(key)
-    if made is None or made[0] is not decay:
-        n = torch.arange(LINEAR_CHUNK_ROWS + 1, dtype=torch.float64, device=decay.device)
-        made = (decay, torch.pow(decay.double()[:, None], n[None, :]).float().contiguous())
-        _POWERS[key] = made
-    return made[1]
+def decay_powers(decay, device) -> torch.Tensor:
+    """float32 [heads, 65]: decay^0 .. decay^64 of every head (`decay`: the heads' numbers), formed in double precision
+    on the host and rounded once: what the chunk kernels multiply scores, outputs and states with."""
+    rows = [[float(d) ** n for n in range(LINEAR_CHUNK_ROWS + 1)] for d in decay]
+    return torch.tensor(rows, dtype=torch.float64).to(torch.float32).to(device).contiguous()
 
 
 def _row_chunks(step, device):

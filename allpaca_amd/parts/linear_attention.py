@@ -59,6 +59,11 @@ class DecayLinearAttention(Mixer):
         self.w_o = ops.prepare_matrix(to_device(tensors[n["o"]], rt), rt.dtype)
         self.norm_w = to_device(tensors[n["norm"]], rt, torch.float32)
         self.decay_t = torch.tensor(self.decay, dtype=torch.float32, device=rt.device)
+        self.powers = None
+        if rt.dtype == torch.bfloat16 and rt.device.type == "cuda":
+            from ..kernels import tuned
+            # (of the float32 decay, which is what the row-by-row kernel multiplies with)
+            self.powers = tuned.decay_powers(self.decay_t.tolist(), rt.device)
 
     def forward(self, h, step, cache) -> torch.Tensor:
         """float32 [rows, hidden]: the mixer's output.  `cache`: the state's view."""
@@ -72,7 +77,7 @@ class DecayLinearAttention(Mixer):
         N = self.H * self.dv
         o = torch.empty((T, N), dtype=torch.float32, device=dev)
         ops.linear_attention(proj, self.q_off, self.k_off, self.v_off, self.H, self.dk, self.dv, self.silu,
-                             self.decay_t, state.state, step, state.slots, o)
+                             self.decay_t, state.state, step, state.slots, o, powers=self.powers)
         a = torch.empty((T, N), dtype=dt, device=dev)
         ops.gated_rmsnorm(o, self.norm_w, self.eps, proj[:, self.g_off:self.g_off + N] if self.gate else None, a)
         out = torch.empty((T, self.D), dtype=torch.float32, device=dev)
